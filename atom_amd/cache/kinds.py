@@ -18,7 +18,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import KVCacheNeed, StateNeed
+from ..parts.base import KVCacheNeed, LatentCacheNeed, StateNeed
 
 
 @dataclass
@@ -29,6 +29,15 @@ class KVBinding:
     group: int
     k_cache: torch.Tensor  # [num_pages, Hkv, page_size, D]
     v_cache: torch.Tensor  # [num_pages, Hkv, D, page_size]
+    writes: bool = True
+
+
+@dataclass
+class LatentBinding:
+    """The pages of one run of a layer that keeps one row per token for all its heads."""
+
+    group: int
+    pages: torch.Tensor    # [num_pages, page_size, width]
     writes: bool = True
 
 
@@ -101,6 +110,27 @@ class PagedKeysValues(CacheKind):
         return KVBinding(binding.group, binding.k_cache, binding.v_cache, writes=False)
 
 
+class PagedLatents(CacheKind):
+    """One row per token in pages, addressed through the same block tables as keys and values."""
+
+    paged = True
+
+    def window(self, need):
+        return need.window
+
+    def keeps_every_token(self, need):
+        return need.window is None
+
+    def page_bytes(self, need, page_size, dtype):
+        return need.width * page_size * _elem_size(dtype)
+
+    def allocate(self, need, *, group, num_pages, page_size, num_slots, device, dtype):
+        return LatentBinding(group, torch.zeros((num_pages, page_size, need.width), dtype=dtype, device=device))
+
+    def share(self, binding):
+        return LatentBinding(binding.group, binding.pages, writes=False)
+
+
 class SlotState(CacheKind):
     def request_bytes(self, need, dtype):
         n = 1
@@ -140,4 +170,5 @@ def kind_of(need) -> CacheKind | None:
 
 
 register_cache_kind(KVCacheNeed, PagedKeysValues())
+register_cache_kind(LatentCacheNeed, PagedLatents())
 register_cache_kind(StateNeed, SlotState())

@@ -179,6 +179,121 @@ class Qwen3Config(ModelConfig):
         return out
 
 
+def _need(raw: dict, key: str, kind, where: str):
+    if not isinstance(raw, dict) or key not in raw or raw[key] is None:
+        raise ConfigError(f"config.json lacks '{key}' in {where}")
+    value = raw[key]
+    if kind is float and isinstance(value, int) and not isinstance(value, bool):
+        value = float(value)
+    if (kind is int and isinstance(value, bool)) or not isinstance(value, kind):
+        raise ConfigError(f"config.json: '{key}' in {where} must be {kind.__name__}, got {value!r}")
+    return value
+
+
+@dataclass(frozen=True)
+class LotoraxConfig(ModelConfig):
+    """``Lotorax``: layers listed one by one, each a mixer (attention over cached latents, or the gated delta
+    rule) and an optional feed-forward (dense, or routed experts) between layer norms; a run of layers may be
+    repeated with the same weights.  config.json keys: ``vocab``, ``width``, ``embedding.scale``, ``norm.eps``,
+    ``layers`` (``type``, ``mixer``, ``mlp``), ``loop`` (``start``, ``stop``, ``times``)."""
+
+    layers: tuple = ()                # the entries of config.json's 'layers', as they are
+    loop: tuple | None = None         # (start, stop, times)
+    norm_eps: float = 1e-5
+    embedding_scale: float = 1.0
+
+    model_type: ClassVar[str] = "lotorax"
+    MIXER_TYPES: ClassVar[tuple] = ("latent_attention", "delta")
+    MLP_KINDS: ClassVar[tuple] = ("dense", "moe")
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "LotoraxConfig":
+        layers = _need(raw, "layers", list, "the model")
+        loop = raw.get("loop")
+        if loop is not None:
+            loop = tuple(_need(loop, k, int, "'loop'") for k in ("start", "stop", "times"))
+        cfg = cls(
+            architecture=raw.get("architecture") or (raw.get("architectures") or ["Lotorax"])[0],
+            vocab_size=_need(raw, "vocab", int, "the model"),
+            hidden_size=_need(raw, "width", int, "the model"),
+            num_hidden_layers=len(layers),
+            # the design names no position limit: angles are formed from positions as they come
+            max_position_embeddings=_take(raw, "max_position_embeddings", int, 1 << 20),
+            tie_word_embeddings=False,
+            torch_dtype=str(raw.get("torch_dtype") or raw.get("dtype") or "bfloat16"),
+            bos_token_id=raw.get("bos_token_id"),
+            eos_token_id=raw.get("eos_token_id"),
+            layers=tuple(layers),
+            loop=loop,
+            norm_eps=_need(raw.get("norm"), "eps", float, "'norm'"),
+            embedding_scale=_need(raw.get("embedding"), "scale", float, "'embedding'"),
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError("norm.eps must be positive")
+        for i, layer in enumerate(self.layers):
+            where = f"layer {i}"
+            kind = _need(layer, "type", str, where)
+            if kind not in self.MIXER_TYPES:
+                raise ConfigError(f"{where}: unknown type {kind!r}; known: {self.MIXER_TYPES}")
+            m = _need(layer, "mixer", dict, where)
+            if kind == "latent_attention":
+                for key in ("heads", "dim", "rot_dim", "vdim", "kv_rank"):
+                    if _need(m, key, int, f"{where}'s mixer") <= 0:
+                        raise ConfigError(f"{where}: {key} must be positive")
+                _need(m, "scale", float, f"{where}'s mixer")
+                rot = _need(m, "rot", dict, f"{where}'s mixer")
+                dims = _need(rot, "dims", int, f"{where}'s rot")
+                _need(rot, "base", float, f"{where}'s rot")
+                if dims % 2 or dims > m["rot_dim"]:
+                    raise ConfigError(f"{where}: rot.dims must be even and at most rot_dim")
+                if rot.get("scaling") is not None:
+                    for key in ("factor", "original", "fast", "slow"):
+                        _need(rot["scaling"], key, float, f"{where}'s rot.scaling")
+            else:
+                for key in ("heads", "kv_heads", "dim", "vdim", "conv"):
+                    if _need(m, key, int, f"{where}'s mixer") <= 0:
+                        raise ConfigError(f"{where}: {key} must be positive")
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
+            mlp = layer.get("mlp")
+            if mlp is not None:
+                mk = _need(mlp, "kind", str, f"{where}'s mlp")
+                if mk not in self.MLP_KINDS:
+                    raise ConfigError(f"{where}: unknown mlp kind {mk!r}; known: {self.MLP_KINDS}")
+                if mk == "dense":
+                    _need(mlp, "ff", int, f"{where}'s mlp")
+                else:
+                    _need(_need(mlp, "expert", dict, f"{where}'s mlp"), "ff", int, f"{where}'s mlp.expert")
+                    router = _need(mlp, "router", dict, f"{where}'s mlp")
+                    if not 0 < _need(router, "top", int, f"{where}'s router") <= _need(router, "experts", int, f"{where}'s router"):
+                        raise ConfigError(f"{where}: the router's top must lie in 1 .. experts")
+        if self.loop is not None:
+            start, stop, times = self.loop
+            if not (0 <= start < stop <= len(self.layers)) or times < 1:
+                raise ConfigError(f"loop {self.loop} does not fit {len(self.layers)} layers")
+
+    def to_dict(self) -> dict:
+        out: dict[str, Any] = {
+            "architecture": self.architecture, "model_type": self.model_type, "vocab": self.vocab_size,
+            "width": self.hidden_size, "embedding": {"scale": self.embedding_scale}, "norm": {"eps": self.norm_eps},
+            "layers": [dict(layer) for layer in self.layers],
+        }
+        if self.loop is not None:
+            out["loop"] = dict(zip(("start", "stop", "times"), self.loop))
+        if self.max_position_embeddings != 1 << 20:
+            out["max_position_embeddings"] = self.max_position_embeddings
+        for key in ("bos_token_id", "eos_token_id"):
+            if getattr(self, key) is not None:
+                out[key] = getattr(self, key)
+        return out
+
+
 def read_config_json(folder: str) -> dict:
     path = os.path.join(folder, "config.json")
     if not os.path.isfile(path):

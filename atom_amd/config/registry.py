@@ -7,7 +7,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable
 
-from .model_config import ConfigError, ModelConfig, Qwen3Config
+from .model_config import ConfigError, LotoraxConfig, ModelConfig, Qwen3Config
 
 
 @dataclass(frozen=True)
@@ -44,6 +44,8 @@ def get_architecture(name: str) -> Architecture:
 
 def model_config_from_dict(raw: dict) -> ModelConfig:
     archs = raw.get("architectures")
+    if not archs and isinstance(raw.get("architecture"), str):
+        archs = [raw["architecture"]]      # a config.json that names its one architecture in the singular
     if not archs:
         raise ConfigError("config.json lacks 'architectures'")
     return get_architecture(archs[0]).config_class.from_dict(raw)
@@ -69,3 +71,7 @@ def _ensure_builtin() -> None:
 
     if "Qwen3ForCausalLM" not in _ARCHITECTURES:
         register_architecture("Qwen3ForCausalLM", Qwen3Config, qwen3_spec)
+    from ..models.lotorax import lotorax_spec
+
+    if "Lotorax" not in _ARCHITECTURES:
+        register_architecture("Lotorax", LotoraxConfig, lotorax_spec)

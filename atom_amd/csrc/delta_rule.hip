@@ -1,0 +1,226 @@
+// The gated delta rule: a recurrent mixer whose state per head is a matrix S [dim, vdim] in float32.
+//
+//   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q          token by token
+//
+// with q and k made unit vectors per head (q also times dim^-1/2), beta = sigmoid(b), and
+// g = exp(-exp(A_log) softplus(a + dt_bias)), all in float32.  Before that, q, k and v pass a short causal
+// convolution over time per channel and SiLU; the convolution's last taps - 1 inputs are carried per request.
+//
+// A request's memory is one float32 row of its state slot: [conv inputs (taps - 1) x channels | S of every head].
+// Requests are walked through the step's device arrays (cu_seqlens_q, slot_of_seq), so the same kernels serve
+// prompt portions, single tokens and padded rows (slot < 0: nothing is read or written) of a replayed graph.
+//
+//   conv_silu_state   one thread per (request, channel) walks the request's tokens of this step
+//   delta_rule        blocks per (request, head, 256 columns); a lane owns one column of S (over dim) in registers, so the
+//                     columns never meet; q, k and the gates of a run of tokens are staged in LDS
+//   delta_out         o / rms(o) * w * silu(gate), rounded to the serving type
+#include "common.h"
+
+constexpr int kMaxTaps = 8;
+
+template <typename TW>
+__global__ void __launch_bounds__(256)
+conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restrict__ taps_w, int taps, int channels,
+                       float* __restrict__ state, long slot_stride, const int* __restrict__ cu_seqlens,
+                       const int* __restrict__ slot_of_seq, float* __restrict__ y) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int seq = blockIdx.y;
+  if (c >= channels) return;
+  const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+  const int slot = slot_of_seq[seq];
+  if (slot < 0) {
+    for (int t = begin; t < end; ++t) y[(size_t)t * channels + c] = 0.f;
+    return;
+  }
+  float w[kMaxTaps], win[kMaxTaps];   // win[taps - 1] is the current input
+#pragma unroll
+  for (int j = 0; j < kMaxTaps; ++j) {
+    w[j] = j < taps ? to_f32(taps_w[(size_t)c * taps + j]) : 0.f;
+    win[j] = 0.f;
+  }
+  float* tail = state + (size_t)slot * slot_stride;   // [taps - 1, channels]
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j)
+    if (j < taps - 1) win[j + 1] = tail[(size_t)j * channels + c];   // shifted down by the first token below
+  for (int t = begin; t < end; ++t) {
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j) win[j] = win[j + 1];
+    const float cur = x[(size_t)t * ldx + c];
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j)
+      if (j == taps - 1) win[j] = cur;
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMaxTaps; ++j)
+      if (j < taps) s = fmaf(w[j], win[j], s);
+    y[(size_t)t * channels + c] = s / (1.f + expf(-s));
+  }
+#pragma unroll
+  for (int j = 0; j < kMaxTaps - 1; ++j)
+    if (j < taps - 1) tail[(size_t)j * channels + c] = win[j + 1];
+}
+
+ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w, int w_dtype, int taps, int channels,
+                                     float* state, long slot_stride, const int* cu_seqlens, const int* slot_of_seq,
+                                     int num_seqs, float* y, hipStream_t stream) {
+  if (taps < 1 || taps > kMaxTaps) return ATOM_TOO_LARGE;
+  if (channels <= 0 || ldx < channels || num_seqs < 0 || slot_stride < (long)(taps - 1) * channels) return ATOM_BAD_SHAPE;
+  if (x == nullptr || taps_w == nullptr || state == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
+  if (num_seqs == 0) return ATOM_OK;
+  if (num_seqs > 65535) return ATOM_TOO_LARGE;
+  dim3 grid((channels + 255) / 256, num_seqs), block(256);
+  ATOM_DISPATCH_DTYPE(w_dtype, hipLaunchKernelGGL((conv_silu_state_kernel<T>), grid, block, 0, stream, x, ldx,
+                                                   (const T*)taps_w, taps, channels, state, slot_stride, cu_seqlens,
+                                                   slot_of_seq, y));
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ the recurrence
+
+constexpr int kRun = 16;   // tokens whose q, k and gates are staged at once
+
+// qkv [T, channels] float32 after convolution and SiLU: q heads (kv_heads x dim) | k heads | v heads (heads x vdim).
+// ab [T, ld_ab] float32: the raw decay inputs at a_off and the raw beta inputs at b_off, one per head.
+template <int DMAX>
+__global__ void __launch_bounds__(256)
+delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab,
+                                  int a_off, int b_off, const float* __restrict__ a_log,
+                                  const float* __restrict__ dt_bias, float* __restrict__ state, long slot_stride,
+                                  long state_off, const int* __restrict__ cu_seqlens,
+                                  const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads,
+                                  int kv_heads, int dim, int vdim) {
+  __shared__ float qs[kRun][DMAX];
+  __shared__ float ks[kRun][DMAX];
+  __shared__ float gs[kRun], bs[kRun];
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int col = blockIdx.z * blockDim.x + tid;   // this lane's column of S
+  const int kvh = head / (heads / kv_heads);
+  const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+  const int slot = slot_of_seq[seq];
+  const bool live = col < vdim;
+  if (slot < 0) {
+    for (int t = begin; t < end; ++t)
+      if (live) out[((size_t)t * heads + head) * vdim + col] = 0.f;
+    return;
+  }
+  float* sp = state + (size_t)slot * slot_stride + state_off + (size_t)head * dim * vdim;   // [dim, vdim]
+  float S[DMAX];
+#pragma unroll
+  for (int i = 0; i < DMAX; ++i) S[i] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
+  const float decay_rate = -expf(a_log[head]);
+  const float bias = dt_bias[head];
+  const float q_scale = rsqrtf((float)dim);
+  const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
+  const int waves = blockDim.x / kWave, wave = tid / kWave, lane = tid % kWave;
+  for (int t0 = begin; t0 < end; t0 += kRun) {
+    const int n = end - t0 < kRun ? end - t0 : kRun;
+    __syncthreads();   // the previous run's q and k have been read
+    // unit vectors: a wave per (token, q or k)
+    for (int item = wave; item < 2 * n; item += waves) {
+      const int j = item >> 1, is_k = item & 1;
+      const float* src = qkv + (size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim;
+      float ss = 0.f;
+      for (int i = lane; i < dim; i += kWave) ss += src[i] * src[i];
+      ss = wave_sum(ss);
+      const float f = (is_k ? 1.f : q_scale) / sqrtf(ss + 1e-6f);
+      float* dst = is_k ? ks[j] : qs[j];
+      for (int i = lane; i < DMAX; i += kWave) dst[i] = i < dim ? src[i] * f : 0.f;
+    }
+    if (tid < n) {
+      const float* r = ab + (size_t)(t0 + tid) * ld_ab;
+      const float z = r[a_off + head] + bias;
+      const float sp_z = z > 20.f ? z : log1pf(expf(z));
+      gs[tid] = expf(decay_rate * sp_z);
+      bs[tid] = 1.f / (1.f + expf(-r[b_off + head]));
+    }
+    __syncthreads();
+    if (live) {
+      for (int j = 0; j < n; ++j) {
+        const float g = gs[j], beta = bs[j];
+        const float v = qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col];
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < DMAX; ++i) {
+          S[i] *= g;
+          dot = fmaf(S[i], ks[j][i], dot);
+        }
+        const float u = beta * (v - dot);
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DMAX; ++i) {
+          S[i] = fmaf(ks[j][i], u, S[i]);
+          o = fmaf(S[i], qs[j][i], o);
+        }
+        out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < dim) sp[(size_t)i * vdim + col] = S[i];
+  }
+}
+
+ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab, int ld_ab, int a_off, int b_off,
+                                const float* a_log, const float* dt_bias, float* state, long slot_stride,
+                                long state_off, const int* cu_seqlens, const int* slot_of_seq, int num_seqs, float* out,
+                                int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || num_seqs < 0) return ATOM_BAD_SHAPE;
+  if (channels != 2 * kv_heads * dim + heads * vdim) return ATOM_BAD_SHAPE;
+  if (a_off < 0 || b_off < 0 || a_off + heads > ld_ab || b_off + heads > ld_ab) return ATOM_BAD_SHAPE;
+  if (state_off < 0 || slot_stride < state_off + (long)heads * dim * vdim) return ATOM_BAD_SHAPE;
+  if (dim > 256 || vdim > 1024) return ATOM_TOO_LARGE;
+  if (num_seqs == 0) return ATOM_OK;
+  if (num_seqs > 65535 || heads > 65535) return ATOM_TOO_LARGE;
+  const int threads = vdim >= 256 ? 256 : (vdim + kWave - 1) / kWave * kWave;
+  dim3 grid(heads, num_seqs, (vdim + threads - 1) / threads), block(threads);
+#define LAUNCH(D)                                                                                                 \
+  hipLaunchKernelGGL((delta_rule_kernel<D>), grid, block, 0, stream, qkv, channels, ab, ld_ab, a_off, b_off, a_log, \
+                     dt_bias, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim, vdim)
+  if (dim <= 32) LAUNCH(32);
+  else if (dim <= 64) LAUNCH(64);
+  else if (dim <= 128) LAUNCH(128);
+  else LAUNCH(256);
+#undef LAUNCH
+  return launch_status();
+}
+
+// ------------------------------------------------------------------ the read-out's norm and gate
+//
+// y[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * w * silu(gate[t, h, :]);  a wave per (token, head)
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ld_gate, int gate_off,
+                 const float* __restrict__ w, float eps, T* __restrict__ y, int heads, int vdim, size_t items) {
+  const size_t item = (size_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  if (item >= items) return;
+  const int lane = threadIdx.x % kWave;
+  const size_t t = item / heads;
+  const int h = (int)(item - t * heads);
+  const float* src = o + item * vdim;
+  const float* gr = gate + t * ld_gate + gate_off + (size_t)h * vdim;
+  float ss = 0.f;
+  for (int i = lane; i < vdim; i += kWave) ss += src[i] * src[i];
+  const float rstd = 1.f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+  T* dst = y + item * vdim;
+  for (int i = lane; i < vdim; i += kWave) {
+    const float g = gr[i];
+    dst[i] = from_f32<T>(src[i] * rstd * w[i] * (g / (1.f + expf(-g))));
+  }
+}
+
+ATOM_EXPORT int atom_delta_out(const float* o, const float* gate, int ld_gate, int gate_off, const float* w, float eps,
+                               void* y, int dtype, int tokens, int heads, int vdim, hipStream_t stream) {
+  if (tokens < 0 || heads <= 0 || vdim <= 0 || gate_off < 0 || gate_off + heads * vdim > ld_gate) return ATOM_BAD_SHAPE;
+  if (o == nullptr || gate == nullptr || w == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
+  const size_t items = (size_t)tokens * heads;
+  if (items == 0) return ATOM_OK;
+  const size_t blocks = (items + 3) / 4;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((delta_out_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, o,
+                                                 gate, ld_gate, gate_off, w, eps, (T*)y, heads, vdim, items));
+  return launch_status();
+}

@@ -31,7 +31,7 @@ def main(argv=None) -> int:
                         help="the most tokens live requests hold at any time (each rounded up to 64)")
     parser.add_argument("--block-size", type=int, default=DEFAULT_PAGE_SIZE,
                         help="tokens a cache page holds")
-    parser.add_argument("--max-requests", type=int, default=8, help="state slots (live requests at a time)")
+    parser.add_argument("--max-requests", type=int, default=4, help="state slots (live requests at a time)")
     parser.add_argument("--enforce-eager", action="store_true", help="never replay captured HIP graphs")
     args = parser.parse_args(argv)
     page_size = args.block_size
@@ -54,8 +54,9 @@ def main(argv=None) -> int:
     say(f"kernel library {ops.path}")
     model, _ = load_model(args.model, dtype=dtype, device=device, progress=say)
     num_pages = max(1, -(-args.max_tokens // page_size))
+    # no request outgrows the pool, so captured graphs size their block tables for that many tokens
     core = build_core(model, ops, dtype=dtype, device=device, page_size=page_size, num_pages=num_pages,
-                      max_num_seqs=args.max_requests,
+                      max_num_seqs=args.max_requests, max_model_len=num_pages * page_size,
                       graph_sizes=None if args.enforce_eager else [1, 2, 4, 8])
     os.makedirs(args.out, exist_ok=True)
     say(f"ready: {num_pages} pages of {page_size} tokens per group, {args.dtype}")

@@ -187,7 +187,10 @@ class HipKernels:
                    "atom_attention_mfma_supports", "atom_attention_decode", "atom_attention_prefill",
                    "atom_attention_prefill_tile_rows", "atom_attention_decode_fused",
                    "atom_attention_decode_fused_supports", "atom_gemm_rows", "atom_gemm_rows_parts",
-                   "atom_gemm_rows_supports", "atom_gemm_tile", "atom_gemm_tile_splits", "atom_gemm_tile_supports"):
+                   "atom_gemm_rows_supports", "atom_gemm_tile", "atom_gemm_tile_splits", "atom_gemm_tile_supports",
+                   "atom_layernorm", "atom_embedding_scaled", "atom_sum_concat", "atom_gated_act", "atom_latent_prepare",
+                   "atom_heads_gemm", "atom_latent_attention", "atom_conv_silu_state", "atom_delta_rule",
+                   "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -830,6 +833,274 @@ class HipKernels:
         gate_up = self.linear(x, weight, bias)
         act = torch.empty((m, inter), dtype=x.dtype, device=x.device)
         return self.silu_mul(gate_up, act)
+
+    # ------------------------------------------------------------------ layer norm and the float32 stream
+
+    _NORM_MODES = {"plain": 0, "init": 1, "add": 2, "post": 3}
+
+    def layernorm(self, x, weight, bias, eps: float, out, residual=None, mode: str = "plain", rows=None,
+                  next_weight=None, next_bias=None):
+        """Layer norm with weight and bias in float32.  mode 'plain': out = LN(x); 'init': residual = x,
+        out = LN(x); 'add': residual += x, out = LN(residual); 'post': residual += LN(x) and then
+        out = LN(residual; next_weight, next_bias) (``out`` None: the sum alone).  With ``rows`` ('plain' and
+        'add') only those source rows are normed and the residual is not written.  ``x`` and ``out`` may have
+        different element types."""
+        x = self.materialize(x)
+        width = x.shape[-1]
+        code = self._NORM_MODES[mode]
+        self._check("norm input", x, (torch.float32, torch.bfloat16), (None, width))
+        self._check("norm weight", weight, torch.float32, (width,))
+        self._check("norm bias", bias, torch.float32, (width,))
+        n_out = rows.numel() if rows is not None else x.shape[0]
+        if out is not None:
+            self._check("norm out", out, (torch.float32, torch.bfloat16), (n_out, width))
+        elif code != 3:
+            raise KernelError("norm: only the 'post' mode may leave out its output")
+        if code:
+            if residual is None:
+                raise KernelError("norm: this mode needs the residual stream")
+            self._check("residual", residual, torch.float32, tuple(x.shape))
+        if rows is not None:
+            if code in (1, 3):
+                raise KernelError("norm: this mode takes all rows")
+            self._check("norm rows", rows, torch.int32, (n_out,))
+        if code == 3 and out is not None:
+            self._check("next norm weight", next_weight, torch.float32, (width,))
+            self._check("next norm bias", next_bias, torch.float32, (width,))
+        self._done("layernorm", self.lib.atom_layernorm(
+            _ptr(x), self._code(x), _ptr(residual), _ptr(weight), _ptr(bias), _ptr(next_weight), _ptr(next_bias),
+            _ptr(out), self._code(out) if out is not None else 0, _ptr(rows), n_out, width, ctypes.c_float(eps), code,
+            self._stream()))
+        return out
+
+    def embedding_scaled(self, table, ids, out, scale: float):
+        """``out = table[ids] * scale`` in float32."""
+        vocab, hidden = table.shape
+        tokens = ids.numel()
+        self._check("embedding table", table, (torch.float32, torch.bfloat16))
+        self._check("token ids", ids, torch.int32, (tokens,))
+        self._check("embedding out", out, torch.float32, (tokens, hidden))
+        self._done("embedding_scaled", self.lib.atom_embedding_scaled(
+            _ptr(table), self._code(table), _ptr(ids), _ptr(out), tokens, hidden, vocab, ctypes.c_float(scale),
+            self._stream()))
+        return out
+
+    def sum_concat(self, hidden, residual, first, out):
+        """``out[t] = [residual[t] + hidden[t] ; first[t]]`` (``residual`` None: hidden alone)."""
+        hidden = self.materialize(hidden)
+        tokens, width = hidden.shape
+        self._check("hidden", hidden, (torch.float32, torch.bfloat16))
+        if residual is not None:
+            self._check("residual", residual, torch.float32, (tokens, width))
+        self._check("first rows", first, torch.float32, (tokens, width))
+        self._check("joined rows", out, (torch.float32, torch.bfloat16), (tokens, 2 * width))
+        self._done("sum_concat", self.lib.atom_sum_concat(
+            _ptr(hidden), self._code(hidden), _ptr(residual), _ptr(first), _ptr(out), self._code(out), tokens, width,
+            self._stream()))
+        return out
+
+    _ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+    def gated_act(self, x, out, activation: str):
+        """``out = act(gate) * up`` for ``x`` = gate | up."""
+        x = self.materialize(x)
+        rows, two = x.shape
+        if two % 2:
+            raise KernelError("gated_act: the input width must be even (gate | up)")
+        if activation not in self._ACTIVATIONS:
+            raise KernelError(f"gated_act: unknown activation {activation!r}; known: {sorted(self._ACTIVATIONS)}")
+        self._check("gated_act input", x, (torch.float32, torch.bfloat16))
+        self._check("gated_act out", out, x.dtype, (rows, two // 2))
+        self._done("gated_act", self.lib.atom_gated_act(_ptr(x), _ptr(out), self._code(out), rows, two // 2,
+                                                        self._ACTIVATIONS[activation], self._stream()))
+        return out
+
+    def linear_f32(self, x, weight, bias=None):
+        """``x @ weight.T (+ bias)`` by float32 multiply-adds whatever the operands' types, float32 out: for the
+        few products that have to be exact (a router's logits)."""
+        x = self.materialize(x)
+        m, k = x.shape
+        n = weight.shape[0]
+        self._check("linear input", x, (torch.float32, torch.bfloat16))
+        self._check("linear weight", weight, (torch.float32, torch.bfloat16), (n, k))
+        if bias is not None:
+            self._check("linear bias", bias, torch.float32, (n,))
+        y = torch.empty((m, n), dtype=torch.float32, device=x.device)
+        self._done("gemm_f32", self.lib.atom_gemm_f32(_ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias),
+                                                      _ptr(y), F32, m, n, k, self._stream()))
+        return y
+
+    # ------------------------------------------------------------------ attention over a cache of latents
+
+    def latent_prepare(self, proj, q_off: int, kv_off: int, heads: int, dim: int, rot: int, rank: int, rot_dims: int,
+                       norm_weight, eps: float, freq, mult: float, positions, slots, pages, q_abs, q_scale: float):
+        """From the float32 product ``proj`` [tokens, *] (queries of ``heads`` x (dim + rot) at ``q_off``, the
+        down-projection of rank + rot at ``kv_off``): the RMS-normed latent and the rotated shared key part go to
+        row ``slots[t]`` of ``pages`` (None: no write), the queries' rotated parts, times ``q_scale``, to
+        ``q_abs[t, h, rank:]``."""
+        tokens, ld = proj.shape
+        width = rank + rot
+        self._check("projections", proj, torch.float32)
+        self._check("latent norm weight", norm_weight, torch.float32, (rank,))
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("absorbed queries", q_abs, (torch.float32, torch.bfloat16), (tokens, heads, width))
+        if rot_dims:
+            self._check("rotation frequencies", freq, torch.float64, (rot_dims // 2,))
+        if slots is not None:
+            self._check("slot mapping", slots, torch.int32, (tokens,))
+            self._check("latent pages", pages, q_abs.dtype, (None, None, width))
+        self._done("latent_prepare", self.lib.atom_latent_prepare(
+            _ptr(proj), ld, q_off, kv_off, heads, dim, rot, rank, rot_dims, _ptr(norm_weight), ctypes.c_float(eps),
+            _ptr(freq) if rot_dims else None, ctypes.c_float(mult), _ptr(positions), _ptr(slots),
+            _ptr(pages) if slots is not None else None, _ptr(q_abs), self._code(q_abs), tokens, ctypes.c_float(q_scale),
+            self._stream()))
+        return q_abs
+
+    def heads_gemm(self, x, x_offset: int, ldx: int, hsx: int, weight, y, y_offset: int, ldy: int, hsy: int, heads: int,
+                   m: int, n: int, k: int, alpha: float = 1.0, gate=None, gate_offset: int = 0, ldg: int = 0):
+        """One small product per head: ``y[t, h, :n] = alpha * x[t, h, :k] @ weight[h].T`` (times
+        ``sigmoid(gate[t, h])`` when given), with ``x`` and ``y`` addressed as flat arrays: element (t, h, i) of x
+        sits at ``x_offset + t * ldx + h * hsx + i``.  ``weight`` is [heads, n, k]."""
+        self._check("per-head input", x, (torch.float32, torch.bfloat16))
+        self._check("per-head weight", weight, (torch.float32, torch.bfloat16), (heads, n, k))
+        self._check("per-head out", y, (torch.float32, torch.bfloat16))
+        if m:
+            if x_offset + (m - 1) * ldx + (heads - 1) * hsx + k > x.numel():
+                raise KernelError("heads_gemm: the input is smaller than its strides say")
+            if y_offset + (m - 1) * ldy + (heads - 1) * hsy + n > y.numel():
+                raise KernelError("heads_gemm: the output is smaller than its strides say")
+        gp = None
+        if gate is not None:
+            self._check("per-head gate", gate, torch.float32)
+            if m and gate_offset + (m - 1) * ldg + heads > gate.numel():
+                raise KernelError("heads_gemm: the gate is smaller than its strides say")
+            gp = ctypes.c_void_p(gate.data_ptr() + 4 * gate_offset)
+        xp = ctypes.c_void_p(x.data_ptr() + x.element_size() * x_offset)
+        yp = ctypes.c_void_p(y.data_ptr() + y.element_size() * y_offset)
+        self._done("heads_gemm", self.lib.atom_heads_gemm(
+            xp, self._code(x), ctypes.c_long(ldx), ctypes.c_long(hsx), _ptr(weight), self._code(weight), yp,
+            self._code(y), ctypes.c_long(ldy), ctypes.c_long(hsy), gp, ctypes.c_long(ldg), heads, m, n, k,
+            ctypes.c_float(alpha), self._stream()))
+        return y
+
+    def latent_attention(self, q_abs, pages, out, meta: AttentionMeta, rank: int, sink=None, window: int | None = None):
+        """Attention of ``q_abs`` [tokens, heads, rank + rot] over pages [num_pages, page_size, rank + rot] whose
+        rows are shared by all heads; the weighted sums of the rows' first ``rank`` entries land in ``out``
+        [tokens, heads, rank].  ``sink`` [heads] joins every softmax's denominator."""
+        tokens, heads, width = q_abs.shape
+        dt = q_abs.dtype
+        self._check("absorbed queries", q_abs, (torch.float32, torch.bfloat16))
+        self._check("latent pages", pages, dt, (None, meta.page_size, width))
+        self._check("attention out", out, dt, (tokens, heads, rank))
+        self._check("token_seq", meta.token_seq, torch.int32, (tokens,))
+        self._check("positions", meta.positions, torch.int32, (tokens,))
+        self._check("block tables", meta.block_tables, torch.int32, (None, None))
+        if sink is not None:
+            self._check("sink", sink, torch.float32, (heads,))
+        if meta.max_context_len > meta.block_tables.shape[1] * meta.page_size:
+            raise KernelError("attention: a context is longer than its block table can name")
+        self._done("latent_attention", self.lib.atom_latent_attention(
+            _ptr(q_abs), _ptr(pages), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions), _ptr(meta.block_tables),
+            meta.block_tables.shape[1], _ptr(sink), self._code(q_abs), tokens, heads, rank, width - rank,
+            meta.page_size, int(window or 0), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ the gated delta rule
+
+    def conv_silu_state(self, x, channels: int, taps_weight, state, cu_seqlens_q, slot_of_seq, out):
+        """Short causal convolution per channel over each request's tokens, then SiLU.  ``x`` float32 [tokens, >=
+        channels] (the first ``channels`` columns are convolved); ``taps_weight`` [channels, taps], last column the
+        current token's; ``state`` float32 [slots, >= (taps - 1) * channels]: a request's last taps - 1 inputs, read
+        and written back.  Requests with slot -1 are padding."""
+        tokens, ldx = x.shape
+        taps = taps_weight.shape[1]
+        seqs = slot_of_seq.numel()
+        self._check("convolution input", x, torch.float32)
+        self._check("taps", taps_weight, (torch.float32, torch.bfloat16), (channels, taps))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("convolution out", out, torch.float32, (tokens, channels))
+        self._done("conv_silu_state", self.lib.atom_conv_silu_state(
+            _ptr(x), ldx, _ptr(taps_weight), self._code(taps_weight), taps, channels, _ptr(state),
+            ctypes.c_long(state.shape[1]), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs, _ptr(out), self._stream()))
+        return out
+
+    def delta_rule(self, qkv, gates, a_off: int, b_off: int, a_log, dt_bias, state, state_off: int, cu_seqlens_q,
+                   slot_of_seq, out, heads: int, kv_heads: int, dim: int, vdim: int):
+        """The gated delta recurrence over each request's tokens.  ``qkv`` float32 [tokens, 2 kv_heads dim + heads
+        vdim] (q | k | v after convolution and SiLU); ``gates`` float32 [tokens, *] with the raw decay inputs at
+        ``a_off`` and the raw beta inputs at ``b_off``; the heads' matrices [heads, dim, vdim] start at
+        ``state_off`` of a slot's row of ``state``.  ``out`` float32 [tokens, heads, vdim]."""
+        tokens, channels = qkv.shape
+        seqs = slot_of_seq.numel()
+        self._check("delta q|k|v", qkv, torch.float32, (tokens, 2 * kv_heads * dim + heads * vdim))
+        self._check("delta gates", gates, torch.float32, (tokens, None))
+        self._check("A_log", a_log, torch.float32, (heads,))
+        self._check("dt_bias", dt_bias, torch.float32, (heads,))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("delta out", out, torch.float32, (tokens, heads, vdim))
+        self._done("delta_rule", self.lib.atom_delta_rule(
+            _ptr(qkv), channels, _ptr(gates), gates.shape[1], a_off, b_off, _ptr(a_log), _ptr(dt_bias), _ptr(state),
+            ctypes.c_long(state.shape[1]), ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
+            _ptr(out), heads, kv_heads, dim, vdim, self._stream()))
+        return out
+
+    def delta_out(self, o, gates, gate_off: int, weight, eps: float, out):
+        """``out[t, h] = o[t, h] / rms(o[t, h]) * weight * silu(gate[t, h])`` with the gate's rows at ``gate_off``
+        of ``gates`` (float32)."""
+        tokens, heads, vdim = o.shape
+        self._check("read-out", o, torch.float32)
+        self._check("gates", gates, torch.float32, (tokens, None))
+        self._check("read-out norm weight", weight, torch.float32, (vdim,))
+        self._check("gated read-out", out, (torch.float32, torch.bfloat16), (tokens, heads * vdim))
+        self._done("delta_out", self.lib.atom_delta_out(
+            _ptr(o), _ptr(gates), gates.shape[1], gate_off, _ptr(weight), ctypes.c_float(eps), _ptr(out),
+            self._code(out), tokens, heads, vdim, self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ routed experts
+
+    def router_choose(self, logits, correction, top: int, renormalize: bool = False):
+        """(ids int32 [tokens, top], weights float32 [tokens, top]) from float32 router logits: scores are
+        sigmoids; the choice adds ``correction`` to them, the weights do not."""
+        tokens, experts = logits.shape
+        self._check("router logits", logits, torch.float32)
+        if correction is not None:
+            self._check("router correction", correction, torch.float32, (experts,))
+        ids = torch.empty((tokens, top), dtype=torch.int32, device=logits.device)
+        weights = torch.empty((tokens, top), dtype=torch.float32, device=logits.device)
+        self._done("router_choose", self.lib.atom_router_choose(
+            _ptr(logits), _ptr(correction), _ptr(ids), _ptr(weights), tokens, experts, top, int(bool(renormalize)),
+            self._stream()))
+        return ids, weights
+
+    def experts_forward(self, x, gate_up, down, ids, weights, activation: str = "silu"):
+        """``sum_k weights[t, k] * down[e] (act(gate[e] x) * (up[e] x))`` with e = ids[t, k].  ``gate_up``
+        [experts, 2 ff, width] (gate rows, then up rows), ``down`` [experts, width, ff]."""
+        x = self.materialize(x)
+        tokens, width = x.shape
+        experts, two_ff, _ = gate_up.shape
+        ff = two_ff // 2
+        top = ids.shape[1]
+        self._check("experts input", x, (torch.float32, torch.bfloat16))
+        self._check("expert gate|up", gate_up, (torch.float32, torch.bfloat16), (experts, 2 * ff, width))
+        self._check("expert down", down, gate_up.dtype, (experts, width, ff))
+        self._check("expert ids", ids, torch.int32, (tokens, top))
+        self._check("expert weights", weights, torch.float32, (tokens, top))
+        if activation not in self._ACTIVATIONS:
+            raise KernelError(f"experts: unknown activation {activation!r}")
+        act = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
+        self._done("experts_gate_up", self.lib.atom_experts_gate_up(
+            _ptr(x), _ptr(gate_up), self._code(gate_up), _ptr(ids), _ptr(act), self._code(x), tokens, top, ff, width,
+            self._ACTIVATIONS[activation], self._stream()))
+        y = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
+        self._done("experts_down", self.lib.atom_experts_down(
+            _ptr(act), _ptr(down), self._code(down), _ptr(ids), _ptr(weights), _ptr(y), self._code(x), tokens, top, ff,
+            width, self._stream()))
+        return y
 
     def sample(self, logits, temperatures, out, top_ks=None, top_ps=None, noise=None, seeds=None, counters=None,
                eps: float = 1e-10):

@@ -10,7 +10,7 @@ from dataclasses import dataclass, field
 
 import torch
 
-from ..parts.base import BLOCKS, EMBEDDINGS, HEADS, NORMS, Part, PartChoice
+from ..parts.base import BLOCKS, EMBEDDINGS, HEADS, JOINS, NORMS, Part, PartChoice
 
 
 @dataclass(frozen=True)
@@ -21,6 +21,7 @@ class LayerRun:
 
     layer: int
     reads_run: int | None = None
+    enters: bool = False   # a pass over repeated layers begins here: the model's join runs before this layer
 
 
 @dataclass
@@ -35,6 +36,10 @@ class ModelSpec:
     embedding: PartChoice = field(default_factory=lambda: PartChoice("token_embedding"))
     head: PartChoice = field(default_factory=lambda: PartChoice("lm_head"))
     order: list[LayerRun] | None = None      # default: every layer once, in turn
+    # what happens to the stream before every run marked ``enters`` (kind from the JOINS registry; built with
+    # hidden_size); it is handed the stream and the embedding's output
+    join: PartChoice | None = None
+    join_prefix: str = "join"
     max_positions: int = 0
     embedding_prefix: str = "model.embed_tokens"
     layer_prefix: str = "model.layers.{}"
@@ -62,7 +67,10 @@ class CausalLM(Part):
         self.head = spec.head.build(HEADS, vocab_size=spec.vocab_size, hidden_size=spec.hidden_size,
                                     tied_to=self.embedding if spec.tie_word_embeddings else None,
                                     prefix=spec.head_prefix)
+        self.join = spec.join.build(JOINS, hidden_size=spec.hidden_size, prefix=spec.join_prefix) if spec.join else None
         self.order = spec.running_order()
+        if self.join is None and any(run.enters for run in self.order):
+            raise ValueError("a run is marked as the start of a pass, but the model names no join")
         for i, run in enumerate(self.order):
             if not (0 <= run.layer < len(self.blocks)):
                 raise ValueError(f"run {i} names layer {run.layer}, the model has {len(self.blocks)}")
@@ -84,7 +92,8 @@ class CausalLM(Part):
         self.device: torch.device | None = None
 
     def children(self):
-        return [self.embedding, *self.blocks, self.final_norm, self.head]
+        return [self.embedding, *([self.join] if self.join is not None else []), *self.blocks, self.final_norm,
+                self.head]
 
     def drops(self, name: str) -> str | None:
         """Why a checkpoint tensor that no parameter names is left aside without an error, or None if it
@@ -113,9 +122,11 @@ class CausalLM(Part):
     def forward(self, ctx, token_ids: torch.Tensor, caches: list, want_rows: torch.Tensor | None):
         """Runs the step's tokens through every run of the order; returns float32 logits
         at ``want_rows`` (None: nothing is wanted, the cache is only filled)."""
-        hidden = self.embedding.forward(ctx, token_ids)
+        hidden = first = self.embedding.forward(ctx, token_ids)
         residual = None
         for run, cache in zip(self.order, caches):
+            if run.enters:
+                hidden, residual = self.join.forward(ctx, hidden, residual, first)
             hidden, residual = self.blocks[run.layer].forward(ctx, hidden, residual, cache)
         if want_rows is None or want_rows.numel() == 0:
             return None

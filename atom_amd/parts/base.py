@@ -11,6 +11,8 @@ configuration, each through a registry of its own (two more, the embedding and t
     position encoding  what a mixer applies to queries and keys (rotary tables)
     block              arranges norm, mixer and feed-forward around the residual stream
 
+An eighth registry, ``JOINS``, holds what a model does to its stream where a pass over repeated layers begins.
+
 A part declares its parameters as ``ParamSpec``s; the loader fills them from checkpoint
 tensors by name (several checkpoint tensors may be stacked into one parameter).
 """
@@ -84,6 +86,10 @@ class Part:
             yield from child.walk()
 
     def full_name(self, local: str) -> str:
+        """The checkpoint name of ``local`` under this part's prefix; an empty ``local`` names the prefix itself
+        (a checkpoint that calls a norm's weight ``l0.norm1`` and its bias ``l0.norm1.b``)."""
+        if not local:
+            return self.prefix
         return f"{self.prefix}.{local}" if self.prefix else local
 
     def finalize(self, device, dtype) -> None:
@@ -102,6 +108,15 @@ class KVCacheNeed:
 
     num_kv_heads: int
     head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class LatentCacheNeed:
+    """A mixer that keeps one row of ``width`` entries per past token, shared by all its heads, in pages (a
+    compressed latent and whatever else every head reads).  ``window`` None = all tokens."""
+
+    width: int
     window: int | None = None
 
 
@@ -194,6 +209,15 @@ class Mixer(Part):
         raise NotImplementedError
 
 
+class Join(Part):
+    """Brings the residual stream and the embedding's output together where a pass over a run of layers begins."""
+
+    def forward(self, ctx, hidden, residual, first):
+        """``hidden`` + ``residual`` is the stream (``residual`` may be None), ``first`` the embedding's output
+        (float32).  Returns (hidden, residual) for the layer that follows."""
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     #: as ``Mixer.accepts_deferred``
     accepts_deferred = False
@@ -253,6 +277,7 @@ POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("head")
+JOINS = Registry("join")
 
 
 @dataclass(frozen=True)

@@ -4,6 +4,8 @@ on its feed-forward output and the residual stream, and the next norm adds them.
 
 from __future__ import annotations
 
+import torch
+
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, PartChoice
 
 
@@ -42,4 +44,55 @@ class PreNormBlock(Block):
         return hidden, residual
 
 
+class SandwichBlock(Block):
+    """Norms before and after each sublayer: ``x += post1(mixer(pre1(x)))``, then ``x += post2(ffn(pre2(x)))``;
+    ``feed_forward`` None leaves the second sublayer out.  As in the pre-norm block, the block hands on its last
+    summand (float32, not yet added) beside the stream, and the norm that follows adds it.  The sum of the mixer's
+    normed output and the norm before the feed-forward are one kernel where the norm offers ``forward_post``."""
+
+    def __init__(self, mixer: PartChoice, feed_forward: PartChoice | None, norm: PartChoice, prefix: str = "",
+                 names: dict[str, str] | None = None):
+        super().__init__(prefix)
+        n = {"mixer_pre": "norm1", "mixer": "mix", "mixer_post": "norm1b", "ffn_pre": "norm2", "ffn": "mlp",
+             "ffn_post": "norm2b", **(names or {})}
+        sub = lambda name: f"{prefix}.{n[name]}" if prefix else n[name]  # noqa: E731
+        self.mixer_pre = norm.build(NORMS, prefix=sub("mixer_pre"))
+        self._mixer = mixer.build(MIXERS, prefix=sub("mixer"))
+        self.mixer_post = norm.build(NORMS, prefix=sub("mixer_post"))
+        self.ffn = feed_forward.build(FEED_FORWARDS, prefix=sub("ffn")) if feed_forward is not None else None
+        self.ffn_pre = norm.build(NORMS, prefix=sub("ffn_pre")) if self.ffn is not None else None
+        self.ffn_post = norm.build(NORMS, prefix=sub("ffn_post")) if self.ffn is not None else None
+
+    @property
+    def mixer(self):
+        return self._mixer
+
+    def children(self):
+        parts = [self.mixer_pre, self._mixer, self.mixer_post]
+        if self.ffn is not None:
+            parts += [self.ffn_pre, self.ffn, self.ffn_post]
+        return parts
+
+    def forward(self, ctx, hidden, residual, cache):
+        ops = ctx.ops
+        if not self.mixer_pre.accepts_deferred:
+            hidden = ops.materialize(hidden)
+        hidden, residual = self.mixer_pre.forward_residual(ctx, hidden, residual)
+        if not self._mixer.accepts_deferred:
+            hidden = ops.materialize(hidden)
+        mixed = ops.materialize(self._mixer.forward(ctx, hidden, cache))
+        if self.ffn is None:
+            return self.mixer_post.forward(ctx, mixed, out_dtype=torch.float32), residual
+        post = getattr(self.mixer_post, "forward_post", None)
+        if post is not None:
+            hidden = post(ctx, mixed, residual, self.ffn_pre)
+        else:
+            hidden, residual = self.ffn_pre.forward_residual(ctx, self.mixer_post.forward(ctx, mixed), residual)
+        if not self.ffn.accepts_deferred:
+            hidden = ops.materialize(hidden)
+        out = ops.materialize(self.ffn.forward(ctx, hidden))
+        return self.ffn_post.forward(ctx, out, out_dtype=torch.float32), residual
+
+
 BLOCKS.register("prenorm", PreNormBlock)
+BLOCKS.register("sandwich", SandwichBlock)

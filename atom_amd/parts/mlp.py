@@ -1,8 +1,10 @@
-"""SiLU-gated dense feed-forward: ``down(silu(gate(x)) * up(x))`` with gate and up in
-one packed product, gate rows first (atom/models/qwen3.py:166-198,321-322;
-atom/model_ops/activation.py:78-82)."""
+"""Gated dense feed-forward: ``down(act(gate(x)) * up(x))`` with gate and up in one packed
+product, gate rows first (atom/models/qwen3.py:166-198,321-322; atom/model_ops/activation.py:78-82).
+SiLU runs the fused gate products; ReLU and tanh-GELU the plain product and an elementwise kernel."""
 
 from __future__ import annotations
+
+import torch
 
 from .base import FEED_FORWARDS, FeedForward, ParamSpec
 
@@ -10,21 +12,25 @@ from .base import FEED_FORWARDS, FeedForward, ParamSpec
 class GatedMLP(FeedForward):
     accepts_deferred = True   # the input goes to the gate/up product as it is
 
+    ACTIVATIONS = ("silu", "relu", "gelu_tanh")
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", bias: bool = False,
-                 prefix: str = "", names: dict[str, str] | None = None):
+                 prefix: str = "", names: dict[str, str] | None = None, weight_suffix: str = ".weight"):
         super().__init__(prefix)
-        if activation != "silu":
-            raise ValueError(f"the gated feed-forward has a SiLU kernel only, got {activation!r}")
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"the gated feed-forward knows the activations {self.ACTIVATIONS}, got {activation!r}")
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        self.activation = activation
         self.bias = bias
         self.names = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj", **(names or {})}
+        self.weight_suffix = weight_suffix   # what a checkpoint appends to a matrix's name ("" : nothing)
 
     def param_specs(self):
-        n, i, h = self.names, self.intermediate_size, self.hidden_size
+        n, i, h, sfx = self.names, self.intermediate_size, self.hidden_size, self.weight_suffix
         specs = {
-            "gate_up.weight": ParamSpec.stacked([(f"{n['gate']}.weight", i), (f"{n['up']}.weight", i)], (h,)),
-            "down.weight": ParamSpec.single(f"{n['down']}.weight", (h, i)),
+            "gate_up.weight": ParamSpec.stacked([(f"{n['gate']}{sfx}", i), (f"{n['up']}{sfx}", i)], (h,)),
+            "down.weight": ParamSpec.single(f"{n['down']}{sfx}", (h, i)),
         }
         if self.bias:
             specs["gate_up.bias"] = ParamSpec.stacked([(f"{n['gate']}.bias", i), (f"{n['up']}.bias", i)], (),
@@ -34,7 +40,13 @@ class GatedMLP(FeedForward):
 
     def forward(self, ctx, x):
         ops = ctx.ops
-        act = ops.linear_silu(x, self.params["gate_up.weight"], self.p("gate_up.bias"))
+        if self.activation == "silu":
+            act = ops.linear_silu(x, self.params["gate_up.weight"], self.p("gate_up.bias"))
+        else:
+            # the fused gate products are SiLU's; any other activation takes the product and one elementwise kernel
+            both = ops.linear(x, self.params["gate_up.weight"], self.p("gate_up.bias"))
+            act = torch.empty((both.shape[0], self.intermediate_size), dtype=both.dtype, device=both.device)
+            ops.gated_act(both, act, self.activation)
         # the down product may come back as slices that the next norm adds while it reads them
         return ops.linear(act, self.params["down.weight"], self.p("down.bias"), defer=True)
 

@@ -1,5 +1,7 @@
 """RMS norm: ``x * rsqrt(mean(x^2) + eps) * w`` in float32, with the residual stream
-(float32) added first when asked.  atom/model_ops/layernorm.py:57-75,450-460."""
+(float32) added first when asked.  atom/model_ops/layernorm.py:57-75,450-460.
+Layer norm (mean taken off, weight and bias) with the same three entry points, and a fourth that
+sums a normed sublayer output into the stream and norms the stream for the next sublayer."""
 
 from __future__ import annotations
 
@@ -50,4 +52,52 @@ class RMSNorm(Norm):
         return ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out, residual=residual, mode=mode, rows=rows)
 
 
+class LayerNorm(Norm):
+    """``(x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b`` in float32, with the residual stream (float32)
+    added first when asked.  ``weight_name`` / ``bias_name`` are the checkpoint's names under the prefix (an
+    empty name: the prefix itself)."""
+
+    def __init__(self, size: int, eps: float, prefix: str = "", weight_name: str = "weight", bias_name: str = "bias"):
+        super().__init__(prefix)
+        self.size = size
+        self.eps = float(eps)
+        self.weight_name, self.bias_name = weight_name, bias_name
+
+    def param_specs(self):
+        return {"weight": ParamSpec.single(self.weight_name, (self.size,), kind="vector", init="one_plus_normal"),
+                "bias": ParamSpec.single(self.bias_name, (self.size,), kind="vector")}
+
+    def forward(self, ctx, x, out_dtype=None):
+        out = torch.empty(tuple(x.shape), dtype=out_dtype or ctx.dtype, device=x.device)
+        return ctx.ops.layernorm(x, self.params["weight"], self.params["bias"], self.eps, out)
+
+    def forward_residual(self, ctx, x, residual):
+        out = torch.empty(tuple(x.shape), dtype=ctx.dtype, device=x.device)
+        if residual is None:
+            residual = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
+            mode = "init"
+        else:
+            mode = "add"
+        ctx.ops.layernorm(x, self.params["weight"], self.params["bias"], self.eps, out, residual=residual, mode=mode)
+        return out, residual
+
+    def forward_post(self, ctx, x, residual, following: "LayerNorm | None"):
+        """The norm of ``x`` joins the residual stream without being rounded on the way, and the stream is
+        normed by ``following`` for the sublayer that comes next (None: the sum alone).  One kernel."""
+        out = None
+        if following is not None:
+            out = torch.empty(tuple(x.shape), dtype=ctx.dtype, device=x.device)
+        ctx.ops.layernorm(x, self.params["weight"], self.params["bias"], self.eps, out, residual=residual, mode="post",
+                          next_weight=following.params["weight"] if following is not None else None,
+                          next_bias=following.params["bias"] if following is not None else None)
+        return out
+
+    def forward_rows(self, ctx, x, residual, rows):
+        out = torch.empty((rows.numel(), self.size), dtype=ctx.dtype, device=x.device)
+        mode = "add" if residual is not None else "plain"
+        return ctx.ops.layernorm(x, self.params["weight"], self.params["bias"], self.eps, out, residual=residual,
+                                 mode=mode, rows=rows)
+
+
 NORMS.register("rmsnorm", RMSNorm)
+NORMS.register("layernorm", LayerNorm)

@@ -8,6 +8,8 @@ is done in float32 by the kernel that also norms q/k and writes the cache.
 
 from __future__ import annotations
 
+import math
+
 import torch
 
 from .base import POSITION_ENCODINGS, PositionEncoding
@@ -40,4 +42,51 @@ class RotaryEncoding(PositionEncoding):
         self.cos, self.sin = _TABLES[key]
 
 
+class ScaledRotary(PositionEncoding):
+    """Rotation of interleaved pairs (2i, 2i + 1) of the first ``dims`` entries by ``position * f_i``, with the
+    frequencies optionally stretched for contexts longer than the ``original`` one (YaRN; Peng et al., "YaRN:
+    Efficient Context Window Extension of Large Language Models"): with ``where(t) = dims * ln(original / (2 pi t))
+    / (2 ln base)``, ``lo = max(floor(where(fast)), 0)``, ``hi = min(ceil(where(slow)), dims - 1)`` and ``ramp_i =
+    clamp((i - lo) / max(hi - lo, 0.001), 0, 1)``, pair i turns at ``f_i / factor * ramp_i + f_i * (1 - ramp_i)``
+    where ``f_i = base^(-2i / dims)``, and cosine and sine are multiplied by ``0.1 ln(factor) + 1``.
+
+    The kernels form angles in float64 from ``freq`` (float64 [dims / 2]), so there is no table over positions and
+    no position limit; ``mult`` is the multiplier of cosine and sine."""
+
+    def __init__(self, dims: int, base: float, factor: float | None = None, original: float | None = None,
+                 fast: float | None = None, slow: float | None = None, prefix: str = ""):
+        super().__init__(prefix)
+        if dims % 2 or dims < 0:
+            raise ValueError(f"rotated dimensions come in pairs, got {dims}")
+        self.dims = int(dims)
+        self.base = float(base)
+        self.scaling = None
+        if factor is not None:
+            if None in (original, fast, slow):
+                raise ValueError("stretched rotation needs factor, original, fast and slow")
+            self.scaling = (float(factor), float(original), float(fast), float(slow))
+        self.freq: torch.Tensor | None = None
+        self.mult = 1.0
+
+    def frequencies(self) -> tuple[torch.Tensor, float]:
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        f = self.base ** (-2.0 * i / max(self.dims, 1))
+        if self.scaling is None:
+            return f, 1.0
+        factor, original, fast, slow = self.scaling
+
+        def where(turns: float) -> float:
+            return self.dims * math.log(original / (2 * math.pi * turns)) / (2 * math.log(self.base))
+
+        lo = max(math.floor(where(fast)), 0)
+        hi = min(math.ceil(where(slow)), self.dims - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / factor * ramp + f * (1 - ramp), 0.1 * math.log(factor) + 1.0
+
+    def finalize(self, device, dtype):
+        freq, self.mult = self.frequencies()
+        self.freq = freq.to(device)
+
+
 POSITION_ENCODINGS.register("rotary", RotaryEncoding)
+POSITION_ENCODINGS.register("scaled_rotary", ScaledRotary)

@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import torch
 
+import plain_lotorax as pl
 from plain_model import causal_attention, exponential_race, rms_norm, rope_neox, silu_and_mul, top_k_top_p_filter
 
 WIDE = torch.float64
@@ -107,6 +108,176 @@ class PlainKernels:
 
     def materialize(self, x):
         return x
+
+    # ---- the kernels of the layer-norm / latent-attention / delta-rule / routed-experts parts
+
+    def layernorm(self, x, weight, bias, eps, out, residual=None, mode="plain", rows=None, next_weight=None,
+                  next_bias=None):
+        xs = x.to(WIDE)
+        w, b = weight.to(WIDE), bias.to(WIDE)
+        if rows is not None:
+            xs = xs[rows.long()]
+        if mode == "post":
+            residual.copy_((residual.to(WIDE) + pl.layer_norm(xs, w, b, eps)).to(torch.float32))
+            if out is not None:
+                out.copy_(pl.layer_norm(residual.to(WIDE), next_weight.to(WIDE), next_bias.to(WIDE), eps).to(out.dtype))
+            return out
+        if mode == "add":
+            res = residual.to(WIDE)
+            xs = xs + (res[rows.long()] if rows is not None else res)
+        if mode in ("init", "add") and rows is None:
+            residual.copy_(xs.to(torch.float32))
+            xs = residual.to(WIDE)
+        out.copy_(pl.layer_norm(xs, w, b, eps).to(out.dtype))
+        return out
+
+    def embedding_scaled(self, table, ids, out, scale):
+        out.copy_((table[ids.long()].to(WIDE) * scale).to(out.dtype))
+        return out
+
+    def sum_concat(self, hidden, residual, first, out):
+        x = hidden.to(WIDE) if residual is None else hidden.to(WIDE) + residual.to(WIDE)
+        out.copy_(torch.cat((x, first.to(WIDE)), dim=-1).to(out.dtype))
+        return out
+
+    def gated_act(self, x, out, activation):
+        g, u = x.to(WIDE).chunk(2, dim=-1)
+        f = {"silu": pl.silu, "relu": torch.relu, "gelu_tanh": pl.gelu_tanh}[activation]
+        out.copy_((f(g) * u).to(out.dtype))
+        return out
+
+    def linear_f32(self, x, weight, bias=None):
+        return self.linear(x, weight, bias, out_dtype=torch.float32)
+
+    def latent_prepare(self, proj, q_off, kv_off, heads, dim, rot, rank, rot_dims, norm_weight, eps, freq, mult,
+                       positions, slots, pages, q_abs, q_scale):
+        T = proj.shape[0]
+        p = proj.to(WIDE)
+        ang = positions.to(WIDE)[:, None] * freq.to(WIDE)[None, :] if rot_dims else None
+
+        def turn(x):   # x [T, ..., rot]
+            if not rot_dims:
+                return x
+            c, s_ = torch.cos(ang) * mult, torch.sin(ang) * mult
+            while c.dim() < x.dim():
+                c, s_ = c.unsqueeze(1), s_.unsqueeze(1)
+            out = x.clone()
+            u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+            out[..., 0:rot_dims:2] = u * c - v * s_
+            out[..., 1:rot_dims:2] = v * c + u * s_
+            return out
+
+        q = p[:, q_off:q_off + heads * (dim + rot)].reshape(T, heads, dim + rot)
+        q_abs[:, :, rank:] = (turn(q[..., dim:]) * q_scale).to(q_abs.dtype)
+        if slots is not None:
+            c = pl.rms_unit(p[:, kv_off:kv_off + rank], eps) * norm_weight.to(WIDE)
+            k = turn(p[:, kv_off + rank:kv_off + rank + rot])
+            flat = pages.view(-1, rank + rot)
+            for t in range(T):
+                if int(slots[t]) >= 0:
+                    flat[int(slots[t])] = torch.cat((c[t], k[t])).to(pages.dtype)
+        return q_abs
+
+    def heads_gemm(self, x, x_offset, ldx, hsx, weight, y, y_offset, ldy, hsy, heads, m, n, k, alpha=1.0, gate=None,
+                   gate_offset=0, ldg=0):
+        xf, yf = x.reshape(-1), y.view(-1)
+        for h in range(heads):
+            xs = torch.as_strided(xf, (m, k), (ldx, 1), x_offset + h * hsx).to(WIDE)
+            r = alpha * (xs @ weight[h].to(WIDE).T)
+            if gate is not None:
+                gv = torch.as_strided(gate.reshape(-1), (m,), (ldg,), gate_offset + h).to(WIDE)
+                r = r * torch.sigmoid(gv)[:, None]
+            torch.as_strided(yf, (m, n), (ldy, 1), y_offset + h * hsy).copy_(r.to(y.dtype))
+        return y
+
+    def latent_attention(self, q_abs, pages, out, meta, rank, sink=None, window=None):
+        tokens, heads, width = q_abs.shape
+        flat = pages.view(-1, width)
+        for t in range(tokens):
+            seq = int(meta.token_seq[t])
+            if seq < 0:
+                out[t] = 0
+                continue
+            pos = int(meta.positions[t])
+            first = max(0, pos - window + 1) if window else 0
+            keys = torch.arange(first, pos + 1)
+            rows = flat[meta.block_tables[seq].long()[keys // meta.page_size] * meta.page_size + keys % meta.page_size].to(WIDE)
+            s = q_abs[t].to(WIDE) @ rows.T                                  # [heads, n]
+            top = s.max(dim=-1, keepdim=True).values
+            if sink is not None:
+                top = torch.maximum(top, sink.to(WIDE)[:, None])
+            e = torch.exp(s - top)
+            denom = e.sum(dim=-1, keepdim=True)
+            if sink is not None:
+                denom = denom + torch.exp(sink.to(WIDE)[:, None] - top)
+            out[t] = ((e / denom) @ rows[:, :rank]).to(out.dtype)
+        return out
+
+    def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out):
+        taps = taps_weight.shape[1]
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            tail = state[slot, :(taps - 1) * channels].view(taps - 1, channels)
+            y, new_tail = pl.short_convolution(x[lo:hi, :channels].to(WIDE), taps_weight.to(WIDE), tail.to(WIDE))
+            out[lo:hi] = pl.silu(y).to(out.dtype)
+            tail.copy_(new_tail.to(tail.dtype))
+        return out
+
+    def delta_rule(self, qkv, gates, a_off, b_off, a_log, dt_bias, state, state_off, cu_seqlens_q, slot_of_seq, out,
+                   heads, kv_heads, dim, vdim):
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            n = hi - lo
+            x = qkv[lo:hi].to(WIDE)
+            q = x[:, :kv_heads * dim].reshape(n, kv_heads, dim)
+            k = x[:, kv_heads * dim:2 * kv_heads * dim].reshape(n, kv_heads, dim)
+            v = x[:, 2 * kv_heads * dim:].reshape(n, heads, vdim)
+            q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
+            k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            gs = gates[lo:hi].to(WIDE)
+            beta = torch.sigmoid(gs[:, b_off:b_off + heads])
+            g = torch.exp(-torch.exp(a_log.to(WIDE)) * pl.softplus(gs[:, a_off:a_off + heads] + dt_bias.to(WIDE)))
+            S = state[slot, state_off:state_off + heads * dim * vdim].view(heads, dim, vdim)
+            for h in range(heads):
+                kv = h // (heads // kv_heads)
+                o, new = pl.delta_rule(q[:, kv], k[:, kv], v[:, h], beta[:, h], g[:, h], S[h].to(WIDE))
+                out[lo:hi, h] = o.to(out.dtype)
+                S[h] = new.to(S.dtype)
+        return out
+
+    def delta_out(self, o, gates, gate_off, weight, eps, out):
+        tokens, heads, vdim = o.shape
+        g = gates[:, gate_off:gate_off + heads * vdim].to(WIDE).view(tokens, heads, vdim)
+        y = pl.rms_unit(o.to(WIDE), eps) * weight.to(WIDE) * pl.silu(g)
+        out.copy_(y.reshape(tokens, heads * vdim).to(out.dtype))
+        return out
+
+    def router_choose(self, logits, correction, top, renormalize=False):
+        s = torch.sigmoid(logits.to(WIDE))
+        pick = s + correction.to(WIDE) if correction is not None else s
+        ids = torch.topk(pick, top, dim=-1).indices
+        w = torch.gather(s, 1, ids)
+        if renormalize:
+            w = w / w.sum(dim=-1, keepdim=True)
+        return ids.to(torch.int32), w.to(torch.float32)
+
+    def experts_forward(self, x, gate_up, down, ids, weights, activation="silu"):
+        f = {"silu": pl.silu, "relu": torch.relu, "gelu_tanh": pl.gelu_tanh}[activation]
+        xs = x.to(WIDE)
+        y = torch.zeros(xs.shape, dtype=WIDE)
+        ff = gate_up.shape[1] // 2
+        for t in range(xs.shape[0]):
+            for k in range(ids.shape[1]):
+                e = int(ids[t, k])
+                both = gate_up[e].to(WIDE) @ xs[t]
+                y[t] += float(weights[t, k]) * (down[e].to(WIDE) @ (f(both[:ff]) * both[ff:]))
+        return y.to(x.dtype)
 
     def exponential_noise(self, seeds, counters, vocab):
         rows = []
