@@ -171,6 +171,15 @@ def routed_choice(h, w, top: int):
     return chosen, torch.gather(s, 1, chosen)
 
 
+def routed_margin(h, w, top: int):
+    """Per token, how far the last chosen expert's choice score lies above the best one left out."""
+    pick = torch.sigmoid(h @ w["router"].T) + w["correction"]
+    if top >= pick.shape[-1]:
+        return torch.full((h.shape[0],), math.inf, dtype=h.dtype)
+    best = torch.topk(pick, top + 1, dim=-1).values
+    return best[:, top - 1] - best[:, top]
+
+
 def routed_ff(h, w, experts: int, top: int):
     chosen, weights = routed_choice(h, w, top)
     out = torch.zeros((h.shape[0], w["e0.down"].shape[0]), dtype=h.dtype)
@@ -200,9 +209,10 @@ def sub(tensors, prefix):
     return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
 
 
-def forward(cfg, tensors, ids, positions=None, carried=None, trail=None):
+def forward(cfg, tensors, ids, positions=None, carried=None, trail=None, margins=None):
     """Logits [T, vocab] of the tokens ``ids`` (one sequence).  ``carried``: what an earlier call returned
-    (then ``positions`` continue); ``trail``: a list that receives the residual stream after every run."""
+    (then ``positions`` continue); ``trail``: a list that receives the residual stream after every run;
+    ``margins``: a list that receives every routed run's ``routed_margin``."""
     tensors = {k: (v.to(F) if v.is_floating_point() else v) for k, v in tensors.items()}
     T = len(ids)
     eps = cfg["norm"]["eps"]
@@ -235,6 +245,8 @@ def forward(cfg, tensors, ids, positions=None, carried=None, trail=None):
                 y = dense_ff(h, w)
             else:
                 y = routed_ff(h, w, layer["mlp"]["router"]["experts"], layer["mlp"]["router"]["top"])
+                if margins is not None:
+                    margins.append(routed_margin(h, w, layer["mlp"]["router"]["top"]))
             x = x + layer_norm(y, tensors[p + "norm2b"], tensors[p + "norm2b.b"], eps)
         if trail is not None:
             trail.append(x)
