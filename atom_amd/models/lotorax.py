@@ -66,7 +66,7 @@ def lotorax_spec(cfg: LotoraxConfig) -> ModelSpec:
     return ModelSpec(
         vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, blocks=blocks, final_norm=norm,
         tie_word_embeddings=False,
-        embedding=PartChoice("scaled_embedding", {"scale": cfg.embedding_scale, "weight_name": ""}),
+        embedding=PartChoice("scaled_f32_embedding", {"scale": cfg.embedding_scale, "weight_name": ""}),
         head=PartChoice("lm_head", {"weight_name": ""}),
         order=lotorax_order(len(cfg.layers), cfg.loop),
         join=PartChoice("concat_projection", {"weight_name": ""}) if cfg.loop is not None else None,

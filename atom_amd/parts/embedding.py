@@ -63,5 +63,5 @@ class LMHead(Head):
 
 
 EMBEDDINGS.register("token_embedding", TokenEmbedding)
-EMBEDDINGS.register("scaled_embedding", ScaledEmbedding)
+EMBEDDINGS.register("scaled_f32_embedding", ScaledEmbedding)
 HEADS.register("lm_head", LMHead)

@@ -246,6 +246,80 @@ def run_long(llm, args, name, raw, layers, gen, batch: int = 16, prompt_len: int
     }
 
 
+# ------------------------------------------------------------------ the Lotorax design beside Qwen3 at equal size
+#
+# Sizes that resemble a real model's layers.  Each names a width and, for both designs, heads of 128; the Lotorax
+# side has four layers (attention over latents + dense, attention + experts, delta rule + dense, attention +
+# experts), the Qwen3 side four layers of the same width with a dense feed-forward of the same size.
+
+def lotorax_pair(size: str) -> tuple[dict, dict]:
+    width, heads, rank, ff, experts, expert_ff, top, vocab = {
+        "1k": (1024, 8, 256, 2816, 16, 704, 2, 32768),
+        "2k": (2048, 16, 512, 5632, 32, 704, 4, 32768),
+        "4k": (4096, 32, 512, 11264, 64, 1408, 4, 65536),
+    }[size]
+    rot = {"base": 1000000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    attn = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": rank, "rot": rot, "scale": 192 ** -0.5}
+    delta = {"heads": heads, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": expert_ff}, "router": {"experts": experts, "top": top}}
+    loto = {"architecture": "Lotorax", "vocab": vocab, "width": width, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5}, "max_position_embeddings": 40960,
+            "layers": [{"type": "latent_attention", "mixer": attn, "mlp": dense},
+                       {"type": "latent_attention", "mixer": attn, "mlp": moe},
+                       {"type": "delta", "mixer": delta, "mlp": dense},
+                       {"type": "latent_attention", "mixer": attn, "mlp": moe}]}
+    qwen = dict(QWEN3_8B, num_hidden_layers=4, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), intermediate_size=ff, vocab_size=vocab)
+    return loto, qwen
+
+
+def run_lotorax(args) -> dict:
+    """Prefill and decode throughput of Lotorax and of Qwen3 at equal size, one engine after the other."""
+    import torch
+
+    from atom_amd import LLMEngine, SamplingParams
+    from atom_amd.config import model_config_from_dict
+
+    out = {"metric": "prefill tok/s and decode tok/s of the Lotorax design beside Qwen3 at equal size (bf16)",
+           "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
+           "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
+           "config": {"batch": args.batch, "context": args.context, "layers": 4}, "sizes": {}}
+    for size in args.lotorax.split(","):
+        row = out["sizes"][size] = {}
+        for name, raw in zip(("lotorax", "qwen3"), lotorax_pair(size)):
+            max_len = max(4096, 2 * args.context)
+            llm = LLMEngine(f"{name}-{size}-random", model_config=model_config_from_dict(raw), load_dummy="random",
+                            seed=5, dtype="bf16", max_model_len=max_len, kv_cache_block_size=16,
+                            num_kvcache_blocks=args.batch * max_len // 16, max_num_seqs=args.batch,
+                            max_num_batched_tokens=16384, enforce_eager=args.enforce_eager,
+                            deferred_output=not args.no_deferred_output,
+                            cudagraph_capture_sizes=[s for s in (1, 2, 4, 8, 16, 32, 64) if s <= args.batch])
+            gen = torch.Generator().manual_seed(5)
+            vocab = raw.get("vocab") or raw["vocab_size"]
+            sp = SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True)
+            times = []
+            for rep in range(3):
+                p = torch.randint(0, vocab, (args.context,), generator=gen).tolist()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                llm.generate([p], sp)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+            elapsed, _ = time_decode(llm, args, {"vocab_size": vocab}, gen, args.batch, args.context, args.steps, args.warmup)
+            row[name] = {"prefill_ms": round(min(times[1:]) * 1e3, 3), "prefill_tok_s": round(args.context / min(times[1:]), 1),
+                         "decode_ms_per_step": round(elapsed / args.steps * 1e3, 4),
+                         "decode_tok_s": round(args.batch * args.steps / elapsed, 1)}
+            print(f"[bench] {size} {name}: {row[name]}", file=sys.stderr, flush=True)
+            release(llm)
+        row["prefill_ratio"] = round(row["lotorax"]["prefill_tok_s"] / row["qwen3"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row["lotorax"]["decode_tok_s"] / row["qwen3"]["decode_tok_s"], 3)
+    first = out["sizes"][args.lotorax.split(",")[0]]["lotorax"]
+    out.update(value=first["decode_tok_s"], ms_per_step=first["decode_ms_per_step"], higher_is_better=True,
+               scaling="weak", vs_baseline=None)
+    return out
+
+
 def make_engine(args, shape_key: str, *, max_seqs: int, max_model_len: int, pages: int, budget: int, layers=None):
     """The engine on a shape's sizes with seeded random weights; returns (engine, name, raw config, layers, generator)."""
     import torch
@@ -491,6 +565,9 @@ def main() -> int:
                          "engine's kernels beside the BLAS library's")
     ap.add_argument("--attention", type=str, default="", metavar="T,C[;T,C]",
                     help="no model: prefill attention alone, T tokens of one request behind C cached ones")
+    ap.add_argument("--lotorax", type=str, default="", metavar="SIZE[,SIZE]",
+                    help="the Lotorax design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
+                         "tokens and decode at --batch, four layers each")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -512,6 +589,9 @@ def main() -> int:
     everything = all(getattr(args, k) == ap.get_default(k) for k in vars(args) if k not in ("gpus", "steps", "warmup"))
     if args.products or args.attention:
         print(json.dumps(run_products(args) if args.products else run_attention(args)), flush=True)
+        return 0
+    if args.lotorax:
+        print(json.dumps(run_lotorax(args)), flush=True)
         return 0
     args.shape = args.shape or "8b"
     line = run_shape(args)
