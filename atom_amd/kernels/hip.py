@@ -190,7 +190,8 @@ class HipKernels:
                    "atom_gemm_rows_supports", "atom_gemm_tile", "atom_gemm_tile_splits", "atom_gemm_tile_supports",
                    "atom_layernorm", "atom_embedding_scaled", "atom_sum_concat", "atom_gated_act", "atom_latent_prepare",
                    "atom_heads_gemm", "atom_latent_attention", "atom_conv_silu_state", "atom_delta_rule",
-                   "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down"):
+                   "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down",
+                   "atom_latent_attention_mfma", "atom_latent_mfma_supports", "atom_latent_mfma_tokens_per_tile"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -214,6 +215,7 @@ class HipKernels:
         self.prefill_key_halves = None
         self.prefill_low_blocks = None   # True / False forces 16 / 32 tokens a wave in the blocks of eight waves
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
+        self.use_mfma_latent = True     # attention over latent pages on the matrix cores (bfloat16, sizes it is built for)
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -983,10 +985,23 @@ class HipKernels:
             ctypes.c_float(alpha), self._stream()))
         return y
 
-    def latent_attention(self, q_abs, pages, out, meta: AttentionMeta, rank: int, sink=None, window: int | None = None):
+    def latent_parts(self, meta: AttentionMeta, heads: int, window: int | None) -> int:
+        """Over how many blocks a row's keys are split in the matrix-core kernel: one for steps with prompt
+        portions (their tiles fill the chip); for single tokens enough blocks to fill it twice, 128 keys each at
+        least."""
+        if meta.max_q_len > 1:
+            return 1
+        blocks = max(1, meta.num_seqs * -(-heads // 64))
+        visible = min(meta.max_context_len, window) if window else meta.max_context_len
+        return max(1, min(-(-2 * self.num_cus // blocks), -(-visible // 128), 64))
+
+    def latent_attention(self, q_abs, pages, out, meta: AttentionMeta, rank: int, sink=None, window: int | None = None,
+                         parts: int | None = None):
         """Attention of ``q_abs`` [tokens, heads, rank + rot] over pages [num_pages, page_size, rank + rot] whose
         rows are shared by all heads; the weighted sums of the rows' first ``rank`` entries land in ``out``
-        [tokens, heads, rank].  ``sink`` [heads] joins every softmax's denominator."""
+        [tokens, heads, rank].  ``sink`` [heads] joins every softmax's denominator.  bfloat16 with sizes the
+        matrix-core kernel is built for runs there (``parts``: blocks a row's keys are split over), anything else
+        the general kernel."""
         tokens, heads, width = q_abs.shape
         dt = q_abs.dtype
         self._check("absorbed queries", q_abs, (torch.float32, torch.bfloat16))
@@ -999,6 +1014,22 @@ class HipKernels:
             self._check("sink", sink, torch.float32, (heads,))
         if meta.max_context_len > meta.block_tables.shape[1] * meta.page_size:
             raise KernelError("attention: a context is longer than its block table can name")
+        if dt == torch.bfloat16 and self.use_mfma_latent and self.lib.atom_latent_mfma_supports(rank, width):
+            self._check("cu_seqlens_q", meta.cu_seqlens_q, torch.int32, (meta.num_seqs + 1,))
+            self._check("context_lens", meta.context_lens, torch.int32, (meta.num_seqs,))
+            if meta.block_tables.shape[0] != meta.num_seqs:
+                raise KernelError("attention: one block table row per request is needed")
+            if parts is None:
+                parts = self.latent_parts(meta, heads, window)
+            ws_o = ws_ml = None
+            if parts > 1:
+                ws_o = self.workspace("latent_o", tokens * heads * parts * rank)
+                ws_ml = self.workspace("latent_ml", tokens * heads * parts * 2)
+            self._done("latent_attention_mfma", self.lib.atom_latent_attention_mfma(
+                _ptr(q_abs), _ptr(pages), _ptr(out), _ptr(ws_o), _ptr(ws_ml), _ptr(meta.cu_seqlens_q),
+                _ptr(meta.context_lens), _ptr(meta.block_tables), meta.block_tables.shape[1], _ptr(sink), meta.num_seqs,
+                tokens, heads, rank, width, meta.page_size, int(window or 0), parts, self._stream()))
+            return out
         self._done("latent_attention", self.lib.atom_latent_attention(
             _ptr(q_abs), _ptr(pages), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions), _ptr(meta.block_tables),
             meta.block_tables.shape[1], _ptr(sink), self._code(q_abs), tokens, heads, rank, width - rank,

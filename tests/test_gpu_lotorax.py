@@ -166,7 +166,8 @@ def _plain_latent_attention(q_abs, rows, rank, sink, positions, window=None):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rank,rot,heads,page,window", [(24, 4, 3, 8, None), (64, 16, 4, 16, None), (40, 8, 2, 4, 37),
-                                                        (128, 32, 6, 16, None)])
+                                                        (128, 32, 6, 16, None), (32, 16, 5, 8, 41), (256, 64, 16, 16, None),
+                                                        (512, 64, 3, 16, None), (48, 8, 70, 4, None)])
 def test_latent_attention_far_keys_page_and_chunk_edges(dtype, rank, rot, heads, page, window):
     """Queries at the first positions, around page borders and around the kernel's chunks of 256 keys, and at the
     end of a long context; key 3 is made to stand out for the last queries, so that a lost far key shows; the sink
@@ -175,7 +176,9 @@ def test_latent_attention_far_keys_page_and_chunk_edges(dtype, rank, rot, heads,
     n = 700
     width = rank + rot
     rows = rnd((n, width), 1, 0.5)
-    positions = [0, 1, 2, page - 1, page, page + 1, 254, 255, 256, 257, 511, 512, 513, n - 2, n - 1]
+    # requests that share one context's pages; each brings a few consecutive tokens that end its own context
+    groups = [[0, 1, 2], [page - 1, page, page + 1], [254, 255, 256, 257], [511, 512, 513], [n - 2, n - 1]]
+    positions = [pos for grp in groups for pos in grp]
     q_abs = rnd((len(positions), heads, width), 2, 0.4)
     rows[3] = 0.1 * rows[3]
     rows[3, :8] = 2.0
@@ -194,14 +197,53 @@ def test_latent_attention_far_keys_page_and_chunk_edges(dtype, rank, rot, heads,
     pages = torch.zeros((num_pages, page, width), dtype=dtype)
     for j in range(n):
         pages[order[j // page], j % page] = rows[j]
-    meta = AttentionMeta(token_seq=i32([0] * len(positions)), positions=i32(positions), block_tables=order.int().view(1, -1).to(DEV),
-                         cu_seqlens_q=i32([0, len(positions)]), context_lens=i32([n]), num_seqs=1, num_tokens=len(positions),
-                         max_q_len=len(positions), max_context_len=n, page_size=page, num_prefill=1)
+    starts = [0]
+    for grp in groups:
+        starts.append(starts[-1] + len(grp))
+    meta = AttentionMeta(token_seq=i32([b for b, grp in enumerate(groups) for _ in grp]), positions=i32(positions),
+                         block_tables=order.int().view(1, -1).repeat(len(groups), 1).contiguous().to(DEV),
+                         cu_seqlens_q=i32(starts), context_lens=i32([grp[-1] + 1 for grp in groups]), num_seqs=len(groups),
+                         num_tokens=len(positions), max_q_len=4, max_context_len=n, page_size=page, num_prefill=len(groups))
     out = torch.empty((len(positions), heads, rank), dtype=dtype, device=DEV)
     ops.latent_attention(q_abs.to(DEV), pages.to(DEV), out, meta, rank, sink.to(DEV), window)
     close(out, want, dtype, "with sink")
     ops.latent_attention(q_abs.to(DEV), pages.to(DEV), out, meta, rank, None, window)
     close(out, _plain_latent_attention(q_abs.double(), rows.double(), rank, None, positions, window), dtype, "no sink")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rank,rot,heads,page", [(64, 16, 4, 16), (128, 32, 6, 8), (40, 8, 2, 4), (512, 64, 16, 16)])
+def test_latent_attention_single_tokens_with_keys_split_over_blocks(dtype, rank, rot, heads, page):
+    """One token a request, contexts of 1 key to 700, a padding row, and a row's keys on one block or split over
+    3 or 8 (the matrix-core kernel; the general kernel takes no split)."""
+    ops = gpu_ops()
+    width = rank + rot
+    contexts = [1, 31, 33, 700, 256, 0, 97]
+    num_pages = sum(-(-c // page) for c in contexts) + 2
+    order = torch.randperm(num_pages, generator=torch.Generator().manual_seed(5)).tolist()
+    pages = torch.zeros((num_pages, page, width), dtype=dtype)
+    tables = torch.zeros((len(contexts), -(-700 // page)), dtype=torch.int32)
+    rows, sink = [], rnd((heads,), 9)
+    for b, c in enumerate(contexts):
+        mine = rnd((c, width), 20 + b, 0.5).to(dtype)
+        rows.append(mine)
+        for j in range(c):
+            if j % page == 0:
+                tables[b, j // page] = order.pop()
+            pages[tables[b, j // page], j % page] = mine[j]
+    q_abs = rnd((len(contexts), heads, width), 3, 0.4).to(dtype)
+    want = torch.zeros((len(contexts), heads, rank), dtype=torch.float64)
+    for b, c in enumerate(contexts):
+        if c:
+            want[b] = _plain_latent_attention(q_abs[b:b + 1].double(), rows[b].double(), rank, sink.double(), [c - 1])[0]
+    meta = AttentionMeta(token_seq=i32([b if c else -1 for b, c in enumerate(contexts)]), positions=i32([max(c - 1, 0) for c in contexts]),
+                         block_tables=tables.to(DEV), cu_seqlens_q=i32(list(range(len(contexts) + 1))),
+                         context_lens=i32(contexts), num_seqs=len(contexts), num_tokens=len(contexts), max_q_len=1,
+                         max_context_len=700, page_size=page, num_prefill=0)
+    for parts in (None, 1, 3, 8):
+        out = torch.full((len(contexts), heads, rank), 7.0, dtype=dtype, device=DEV)
+        ops.latent_attention(q_abs.to(DEV), pages.to(DEV), out, meta, rank, sink.to(DEV), None, parts=parts)
+        close(out, want, dtype, f"parts {parts}")
 
 
 # ------------------------------------------------------------------ the delta rule
