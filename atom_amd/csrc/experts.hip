@@ -154,3 +154,232 @@ ATOM_EXPORT int atom_experts_down(const void* act_in, const void* w, int w_dtype
 #undef LAUNCH
   return launch_status();
 }
+
+// ------------------------------------------------------------------ many tokens: pairs sorted by expert, grouped products
+//
+//   experts_sort      one block: counts the pairs of every expert, gives each expert whole tiles of 64 rows
+//                     (padded), and every pair its row.  tile_expert[tile] = expert or -1; row_pair[row] = pair or
+//                     -1; pair_row[pair] = row.  Rows of one expert come in no fixed order; a row's result does
+//                     not depend on its place.
+//   grouped_gate_up   act[row] = f(W_gate[e] x) * (W_up[e] x) for the rows of a tile, on the matrix cores.  The
+//                     weights are the A operand and the tokens the B operand, both read straight from memory in
+//                     16-byte pieces, so a lane ends up with four consecutive columns of one row.
+//   grouped_down      y[row] = W_down[e] act[row], float32
+//   experts_combine   out[t] = sum_k weight[t, k] * y[pair_row[t, k]], in the order of k
+//
+// bfloat16 only; width and ff multiples of 8.
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+constexpr int kTileRows = 64;
+
+__global__ void __launch_bounds__(1024)
+experts_sort_kernel(const int* __restrict__ ids, int pairs, int experts, int max_tiles, int* __restrict__ tile_expert,
+                    int* __restrict__ row_pair, int* __restrict__ pair_row) {
+  extern __shared__ int sm[];   // counts [experts], first row of each expert [experts]
+  int* counts = sm;
+  int* first = sm + experts;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < experts; e += 1024) counts[e] = 0;
+  for (int i = tid; i < max_tiles; i += 1024) tile_expert[i] = -1;
+  for (int i = tid; i < max_tiles * kTileRows; i += 1024) row_pair[i] = -1;
+  __syncthreads();
+  for (int i = tid; i < pairs; i += 1024) atomicAdd(&counts[ids[i]], 1);
+  __syncthreads();
+  if (tid == 0) {
+    int tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = tile * kTileRows;
+      const int n = (counts[e] + kTileRows - 1) / kTileRows;
+      for (int j = 0; j < n; ++j) tile_expert[tile + j] = e;
+      tile += n;
+      counts[e] = 0;   // now the fill level
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < pairs; i += 1024) {
+    const int e = ids[i];
+    const int row = first[e] + atomicAdd(&counts[e], 1);
+    row_pair[row] = i;
+    pair_row[i] = row;
+  }
+}
+
+__device__ __forceinline__ bf16x8 load8(const bf16_t* p, bool ok) {
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? *reinterpret_cast<const bf16x8*>(p) : zero;
+}
+
+// grid (tiles, ceil(ff / 64)); block 256 = 2 x 2 waves; a wave owns 32 rows x 32 columns of gate and of up
+__global__ void __launch_bounds__(256)
+grouped_gate_up_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const int* __restrict__ tile_expert,
+                       const int* __restrict__ row_pair, bf16_t* __restrict__ act_out, int top, int ff, int width,
+                       int act) {
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave, r = lane % 16, g = lane / 16;
+  const int row0 = tile * kTileRows + (wave / 2) * 32;
+  const int col0 = blockIdx.y * 64 + (wave % 2) * 32;
+  const bf16_t* we = w + (size_t)e * 2 * ff * width;
+  const bf16_t* xrow[2];
+  bool xok[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int pair = row_pair[row0 + rt * 16 + r];
+    xok[rt] = pair >= 0;
+    xrow[rt] = x + (size_t)(pair >= 0 ? pair / top : 0) * width;
+  }
+  const bf16_t* grow[2];
+  const bf16_t* urow[2];
+  bool cok[2];
+#pragma unroll
+  for (int ct = 0; ct < 2; ++ct) {
+    const int col = col0 + ct * 16 + r;
+    cok[ct] = col < ff;
+    grow[ct] = we + (size_t)(cok[ct] ? col : 0) * width;
+    urow[ct] = we + (size_t)(ff + (cok[ct] ? col : 0)) * width;
+  }
+  f32x4 ga[2][2], ua[2][2];
+#pragma unroll
+  for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) ga[ct][rt] = ua[ct][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < width; k0 += 32) {
+    const int k = k0 + 8 * g;
+    const bool kok = k < width;
+    bf16x8 xb[2], gw[2], uw[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) xb[rt] = load8(xrow[rt] + k, kok && xok[rt]);
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      gw[ct] = load8(grow[ct] + k, kok && cok[ct]);
+      uw[ct] = load8(urow[ct] + k, kok && cok[ct]);
+    }
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) {
+        ga[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gw[ct], xb[rt], ga[ct][rt], 0, 0, 0);
+        ua[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uw[ct], xb[rt], ua[ct][rt], 0, 0, 0);
+      }
+  }
+  // lane (r, g) holds columns col0 + ct * 16 + 4g .. + 3 of row row0 + rt * 16 + r
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int row = row0 + rt * 16 + r;
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const int col = col0 + ct * 16 + 4 * g;
+      if (col + 3 < ff) {
+        bf16x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = static_cast<__bf16>(expert_activation(ga[ct][rt][i], act) * ua[ct][rt][i]);
+        *reinterpret_cast<bf16x4*>(act_out + (size_t)row * ff + col) = o;
+      } else {
+        for (int i = 0; i < 4; ++i)
+          if (col + i < ff)
+            act_out[(size_t)row * ff + col + i] = static_cast<bf16_t>(expert_activation(ga[ct][rt][i], act) * ua[ct][rt][i]);
+      }
+    }
+  }
+}
+
+// grid (tiles, ceil(width / 128)); block 256 = 2 x 2 waves; a wave owns 32 rows x 64 columns
+__global__ void __launch_bounds__(256)
+grouped_down_kernel(const bf16_t* __restrict__ act_in, const bf16_t* __restrict__ w, const int* __restrict__ tile_expert,
+                    float* __restrict__ y, int ff, int width) {
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave, r = lane % 16, g = lane / 16;
+  const int row0 = tile * kTileRows + (wave / 2) * 32;
+  const int col0 = blockIdx.y * 128 + (wave % 2) * 64;
+  const bf16_t* we = w + (size_t)e * width * ff;
+  const bf16_t* arow[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) arow[rt] = act_in + (size_t)(row0 + rt * 16 + r) * ff;
+  const bf16_t* wrow[4];
+  bool cok[4];
+#pragma unroll
+  for (int ct = 0; ct < 4; ++ct) {
+    const int col = col0 + ct * 16 + r;
+    cok[ct] = col < width;
+    wrow[ct] = we + (size_t)(cok[ct] ? col : 0) * ff;
+  }
+  f32x4 acc[4][2];
+#pragma unroll
+  for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) acc[ct][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < ff; k0 += 32) {
+    const int k = k0 + 8 * g;
+    const bool kok = k < ff;
+    bf16x8 ab[2], wa[4];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) ab[rt] = load8(arow[rt] + k, kok);
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) wa[ct] = load8(wrow[ct] + k, kok && cok[ct]);
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) acc[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ct], ab[rt], acc[ct][rt], 0, 0, 0);
+  }
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int row = row0 + rt * 16 + r;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct) {
+      const int col = col0 + ct * 16 + 4 * g;
+      if (col + 3 < width) {
+        *reinterpret_cast<f32x4*>(y + (size_t)row * width + col) = acc[ct][rt];
+      } else {
+        for (int i = 0; i < 4; ++i)
+          if (col + i < width) y[(size_t)row * width + col + i] = acc[ct][rt][i];
+      }
+    }
+  }
+}
+
+__global__ void experts_combine_kernel(const float* __restrict__ y, const int* __restrict__ pair_row,
+                                       const float* __restrict__ weights, bf16_t* __restrict__ out, int top, int width) {
+  const size_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) total += weights[t * top + k] * y[(size_t)pair_row[t * top + k] * width + c];
+    out[t * width + c] = static_cast<bf16_t>(total);
+  }
+}
+
+// Rows of the padded, sorted layout for `pairs` pairs over `experts` experts (an upper bound, in whole tiles).
+ATOM_EXPORT int atom_experts_grouped_tiles(int pairs, int experts) { return pairs / kTileRows + experts; }
+
+ATOM_EXPORT int atom_experts_grouped_supports(int ff, int width, int experts) {
+  return ff > 0 && width > 0 && ff % 8 == 0 && width % 8 == 0 && experts > 0 && experts <= 4096;
+}
+
+// x [tokens, width] bf16; gate_up [experts, 2 ff, width]; down [experts, width, ff]; ids, weights [tokens, top];
+// scratch: tile_expert [tiles], row_pair [tiles * 64], pair_row [tokens * top] (int32), act [tiles * 64, ff] bf16
+// (rows of padding are never read for a live row), y [tiles * 64, width] float32; out [tokens, width] bf16.
+ATOM_EXPORT int atom_experts_grouped(const void* x, const void* gate_up, const void* down, const int* ids,
+                                     const float* weights, int* tile_expert, int* row_pair, int* pair_row, void* act_buf,
+                                     float* y, void* out, int tokens, int top, int experts, int ff, int width, int act,
+                                     hipStream_t stream) {
+  if (tokens < 0 || top <= 0 || act < 0 || act > 2) return ATOM_BAD_SHAPE;
+  if (!atom_experts_grouped_supports(ff, width, experts)) return ATOM_UNSUPPORTED;
+  if (tokens == 0) return ATOM_OK;
+  const int pairs = tokens * top;
+  const int tiles = atom_experts_grouped_tiles(pairs, experts);
+  if (tiles > 0x7fffffff / kTileRows) return ATOM_TOO_LARGE;
+  hipLaunchKernelGGL(experts_sort_kernel, dim3(1), dim3(1024), 2 * experts * sizeof(int), stream, ids, pairs, experts,
+                     tiles, tile_expert, row_pair, pair_row);
+  hipLaunchKernelGGL(grouped_gate_up_kernel, dim3(tiles, (ff + 63) / 64), dim3(256), 0, stream, (const bf16_t*)x,
+                     (const bf16_t*)gate_up, tile_expert, row_pair, (bf16_t*)act_buf, top, ff, width, act);
+  hipLaunchKernelGGL(grouped_down_kernel, dim3(tiles, (width + 127) / 128), dim3(256), 0, stream, (const bf16_t*)act_buf,
+                     (const bf16_t*)down, tile_expert, y, ff, width);
+  hipLaunchKernelGGL(experts_combine_kernel, dim3(tokens), dim3(256), 0, stream, y, pair_row, weights, (bf16_t*)out, top,
+                     width);
+  return launch_status();
+}

@@ -191,7 +191,8 @@ class HipKernels:
                    "atom_layernorm", "atom_embedding_scaled", "atom_sum_concat", "atom_gated_act", "atom_latent_prepare",
                    "atom_heads_gemm", "atom_latent_attention", "atom_conv_silu_state", "atom_delta_rule",
                    "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down",
-                   "atom_latent_attention_mfma", "atom_latent_mfma_supports", "atom_latent_mfma_tokens_per_tile"):
+                   "atom_latent_attention_mfma", "atom_latent_mfma_supports", "atom_latent_mfma_tokens_per_tile",
+                   "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -216,6 +217,9 @@ class HipKernels:
         self.prefill_low_blocks = None   # True / False forces 16 / 32 tokens a wave in the blocks of eight waves
         self.use_fused_decode = True    # decode-only steps of few rows: norm, rotation and cache write inside attention
         self.use_mfma_latent = True     # attention over latent pages on the matrix cores (bfloat16, sizes it is built for)
+        # routed experts: from this many (token, choice) pairs on, the pairs are sorted by expert and run as grouped
+        # products on the matrix cores; below, every pair reads its expert's rows itself
+        self.grouped_experts_from = 64
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -1123,6 +1127,18 @@ class HipKernels:
         self._check("expert weights", weights, torch.float32, (tokens, top))
         if activation not in self._ACTIVATIONS:
             raise KernelError(f"experts: unknown activation {activation!r}")
+        if (x.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and tokens * top >= self.grouped_experts_from
+                and self.lib.atom_experts_grouped_supports(ff, width, experts)):
+            tiles = self.lib.atom_experts_grouped_tiles(tokens * top, experts)
+            ints = self.workspace("experts_ints", tiles * 65 + tokens * top, torch.int32)
+            act = self.workspace("experts_act", tiles * 64 * ff, torch.bfloat16)
+            rows = self.workspace("experts_rows", tiles * 64 * width)
+            y = torch.empty((tokens, width), dtype=x.dtype, device=x.device)
+            self._done("experts_grouped", self.lib.atom_experts_grouped(
+                _ptr(x), _ptr(gate_up), _ptr(down), _ptr(ids), _ptr(weights), _ptr(ints),
+                ctypes.c_void_p(ints.data_ptr() + 4 * tiles), ctypes.c_void_p(ints.data_ptr() + 4 * tiles * 65), _ptr(act),
+                _ptr(rows), _ptr(y), tokens, top, experts, ff, width, self._ACTIVATIONS[activation], self._stream()))
+            return y
         act = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
         self._done("experts_gate_up", self.lib.atom_experts_gate_up(
             _ptr(x), _ptr(gate_up), self._code(gate_up), _ptr(ids), _ptr(act), self._code(x), tokens, top, ff, width,

@@ -351,7 +351,8 @@ def test_router_choice_uses_the_correction_for_the_choice_only(experts, top):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,ff,experts,top,tokens", [(48, 40, 5, 2, 13), (40, 16, 6, 3, 1), (64, 32, 8, 1, 70)])
+@pytest.mark.parametrize("width,ff,experts,top,tokens", [(48, 40, 5, 2, 13), (40, 16, 6, 3, 1), (64, 32, 8, 1, 70),
+                                                         (48, 40, 5, 2, 300), (136, 72, 33, 4, 129), (256, 96, 12, 2, 64)])
 def test_experts_forward(dtype, width, ff, experts, top, tokens):
     ops = gpu_ops()
     x = rnd((tokens, width), 1).to(dtype)
