@@ -11,8 +11,9 @@
 // prompt portions, single tokens and padded rows (slot < 0: nothing is read or written) of a replayed graph.
 //
 //   conv_silu_state   one thread per (request, channel) walks the request's tokens of this step
-//   delta_rule        blocks per (request, head, 256 columns); a lane owns one column of S (over dim) in registers, so the
-//                     columns never meet; q, k and the gates of a run of tokens are staged in LDS
+//   delta_rule        blocks per (request, head, group of columns); a column of S (over dim) sits in the registers of up
+//                     to 16 adjacent lanes, so the columns never meet; q, k and the gates of a run of tokens are
+//                     staged in LDS
 //   delta_out         o / rms(o) * w * silu(gate), rounded to the serving type
 #include "common.h"
 
@@ -78,46 +79,53 @@ ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w
 // ------------------------------------------------------------------ the recurrence
 
 constexpr int kRun = 16;   // tokens whose q, k and gates are staged at once
+constexpr int kDPL = 16;   // entries of a column of S that one lane holds
 
 // qkv [T, channels] float32 after convolution and SiLU: q heads (kv_heads x dim) | k heads | v heads (heads x vdim).
 // ab [T, ld_ab] float32: the raw decay inputs at a_off and the raw beta inputs at b_off, one per head.
-template <int DMAX>
+// A column of S (dim entries) is spread over LPC adjacent lanes, entry i in lane i % LPC, so that a token costs each
+// lane 16 entries and two sums over the LPC lanes; the sums over a lane's entries run in four independent chains.
+template <int LPC>
 __global__ void __launch_bounds__(256)
-delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab,
-                                  int a_off, int b_off, const float* __restrict__ a_log,
-                                  const float* __restrict__ dt_bias, float* __restrict__ state, long slot_stride,
-                                  long state_off, const int* __restrict__ cu_seqlens,
-                                  const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads,
-                                  int kv_heads, int dim, int vdim) {
+delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab, int a_off,
+                  int b_off, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                  float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
+                  const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads, int kv_heads, int dim,
+                  int vdim) {
+  constexpr int DMAX = kDPL * LPC;
   __shared__ float qs[kRun][DMAX];
   __shared__ float ks[kRun][DMAX];
   __shared__ float gs[kRun], bs[kRun];
   const int head = blockIdx.x, seq = blockIdx.y;
   const int tid = threadIdx.x;
-  const int col = blockIdx.z * blockDim.x + tid;   // this lane's column of S
+  const int sub = tid % LPC;
+  const int col = blockIdx.z * (256 / LPC) + tid / LPC;   // this lane's column of S
   const int kvh = head / (heads / kv_heads);
   const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
   const int slot = slot_of_seq[seq];
   const bool live = col < vdim;
   if (slot < 0) {
     for (int t = begin; t < end; ++t)
-      if (live) out[((size_t)t * heads + head) * vdim + col] = 0.f;
+      if (live && sub == 0) out[((size_t)t * heads + head) * vdim + col] = 0.f;
     return;
   }
   float* sp = state + (size_t)slot * slot_stride + state_off + (size_t)head * dim * vdim;   // [dim, vdim]
-  float S[DMAX];
+  float S[kDPL];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
+  for (int j = 0; j < kDPL; ++j) {
+    const int i = j * LPC + sub;
+    S[j] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
+  }
   const float decay_rate = -expf(a_log[head]);
   const float bias = dt_bias[head];
-  const float q_scale = rsqrtf((float)dim);
+  const float q_scale = 1.f / sqrtf((float)dim);
   const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
-  const int waves = blockDim.x / kWave, wave = tid / kWave, lane = tid % kWave;
+  const int wave = tid / kWave, lane = tid % kWave;
   for (int t0 = begin; t0 < end; t0 += kRun) {
     const int n = end - t0 < kRun ? end - t0 : kRun;
     __syncthreads();   // the previous run's q and k have been read
     // unit vectors: a wave per (token, q or k)
-    for (int item = wave; item < 2 * n; item += waves) {
+    for (int item = wave; item < 2 * n; item += 4) {
       const int j = item >> 1, is_k = item & 1;
       const float* src = qkv + (size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim;
       float ss = 0.f;
@@ -135,31 +143,35 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       bs[tid] = 1.f / (1.f + expf(-r[b_off + head]));
     }
     __syncthreads();
-    if (live) {
-      for (int j = 0; j < n; ++j) {
-        const float g = gs[j], beta = bs[j];
-        const float v = qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col];
-        float dot = 0.f;
+    for (int j = 0; j < n; ++j) {
+      const float g = gs[j], beta = bs[j];
+      const float v = live ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < DMAX; ++i) {
-          S[i] *= g;
-          dot = fmaf(S[i], ks[j][i], dot);
-        }
-        const float u = beta * (v - dot);
-        float o = 0.f;
-#pragma unroll
-        for (int i = 0; i < DMAX; ++i) {
-          S[i] = fmaf(ks[j][i], u, S[i]);
-          o = fmaf(S[i], qs[j][i], o);
-        }
-        out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
+      for (int e = 0; e < kDPL; ++e) {
+        S[e] *= g;
+        part[e & 3] = fmaf(S[e], ks[j][e * LPC + sub], part[e & 3]);
       }
+      float dot = (part[0] + part[1]) + (part[2] + part[3]);
+#pragma unroll
+      for (int off = 1; off < LPC; off <<= 1) dot += __shfl_xor(dot, off, kWave);
+      const float u = beta * (v - dot);
+      part[0] = part[1] = part[2] = part[3] = 0.f;
+#pragma unroll
+      for (int e = 0; e < kDPL; ++e) {
+        S[e] = fmaf(ks[j][e * LPC + sub], u, S[e]);
+        part[e & 3] = fmaf(S[e], qs[j][e * LPC + sub], part[e & 3]);
+      }
+      float o = (part[0] + part[1]) + (part[2] + part[3]);
+#pragma unroll
+      for (int off = 1; off < LPC; off <<= 1) o += __shfl_xor(o, off, kWave);
+      if (live && sub == 0) out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
     }
   }
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < dim) sp[(size_t)i * vdim + col] = S[i];
+  for (int j = 0; j < kDPL; ++j) {
+    const int i = j * LPC + sub;
+    if (live && i < dim) sp[(size_t)i * vdim + col] = S[j];
   }
 }
 
@@ -171,18 +183,24 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
   if (channels != 2 * kv_heads * dim + heads * vdim) return ATOM_BAD_SHAPE;
   if (a_off < 0 || b_off < 0 || a_off + heads > ld_ab || b_off + heads > ld_ab) return ATOM_BAD_SHAPE;
   if (state_off < 0 || slot_stride < state_off + (long)heads * dim * vdim) return ATOM_BAD_SHAPE;
-  if (dim > 256 || vdim > 1024) return ATOM_TOO_LARGE;
+  if (dim > 256) return ATOM_TOO_LARGE;
   if (num_seqs == 0) return ATOM_OK;
   if (num_seqs > 65535 || heads > 65535) return ATOM_TOO_LARGE;
-  const int threads = vdim >= 256 ? 256 : (vdim + kWave - 1) / kWave * kWave;
-  dim3 grid(heads, num_seqs, (vdim + threads - 1) / threads), block(threads);
-#define LAUNCH(D)                                                                                                 \
-  hipLaunchKernelGGL((delta_rule_kernel<D>), grid, block, 0, stream, qkv, channels, ab, ld_ab, a_off, b_off, a_log, \
+  int lpc = 1;
+  while (lpc * kDPL < dim) lpc *= 2;
+  const int cols = 256 / lpc;
+  dim3 grid(heads, num_seqs, (vdim + cols - 1) / cols), block(256);
+  if (grid.z > 65535) return ATOM_TOO_LARGE;
+#define LAUNCH(L)                                                                                                 \
+  hipLaunchKernelGGL((delta_rule_kernel<L>), grid, block, 0, stream, qkv, channels, ab, ld_ab, a_off, b_off, a_log, \
                      dt_bias, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim, vdim)
-  if (dim <= 32) LAUNCH(32);
-  else if (dim <= 64) LAUNCH(64);
-  else if (dim <= 128) LAUNCH(128);
-  else LAUNCH(256);
+  switch (lpc) {
+    case 1: LAUNCH(1); break;
+    case 2: LAUNCH(2); break;
+    case 4: LAUNCH(4); break;
+    case 8: LAUNCH(8); break;
+    default: LAUNCH(16); break;
+  }
 #undef LAUNCH
   return launch_status();
 }

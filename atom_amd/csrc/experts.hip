@@ -60,6 +60,7 @@ __device__ __forceinline__ float expert_activation(float g, int act) {
 }
 
 constexpr int kExpCols = 32;   // output columns of a block: 4 waves x 8
+typedef __attribute__((ext_vector_type(8))) __bf16 ex_bf16x8;
 
 template <typename T, typename TW>
 __global__ void __launch_bounds__(256)
@@ -80,10 +81,28 @@ experts_gate_up_kernel(const T* __restrict__ x, const TW* __restrict__ w, const 
     const TW* gr = we + (size_t)col * width;
     const TW* ur = we + (size_t)(ff + col) * width;
     float g = 0.f, u = 0.f;
-    for (int i = lane; i < width; i += kWave) {
-      const float xv = xs[i];
-      g = fmaf(xv, to_f32(gr[i]), g);
-      u = fmaf(xv, to_f32(ur[i]), u);
+    if constexpr (sizeof(TW) == 2) {
+      if (width % 8 == 0) {   // 16 bytes a lane and row
+        for (int i = lane * 8; i < width; i += kWave * 8) {
+          const ex_bf16x8 gv = *reinterpret_cast<const ex_bf16x8*>(gr + i), uv = *reinterpret_cast<const ex_bf16x8*>(ur + i);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            g = fmaf(xs[i + e], static_cast<float>(gv[e]), g);
+            u = fmaf(xs[i + e], static_cast<float>(uv[e]), u);
+          }
+        }
+      } else {
+        for (int i = lane; i < width; i += kWave) {
+          g = fmaf(xs[i], to_f32(gr[i]), g);
+          u = fmaf(xs[i], to_f32(ur[i]), u);
+        }
+      }
+    } else {
+      for (int i = lane; i < width; i += kWave) {
+        const float xv = xs[i];
+        g = fmaf(xv, to_f32(gr[i]), g);
+        u = fmaf(xv, to_f32(ur[i]), u);
+      }
     }
     g = wave_sum(g);
     u = wave_sum(u);
@@ -108,7 +127,19 @@ experts_down_kernel(const T* __restrict__ act_in, const TW* __restrict__ w, cons
       const int e = ids[(size_t)t * top + k];
       const TW* wr = w + ((size_t)e * width + col) * ff;
       float s = 0.f;
-      for (int i = lane; i < ff; i += kWave) s = fmaf(as[k * ff + i], to_f32(wr[i]), s);
+      bool done = false;
+      if constexpr (sizeof(TW) == 2) {
+        if (ff % 8 == 0) {
+          for (int i = lane * 8; i < ff; i += kWave * 8) {
+            const ex_bf16x8 wv = *reinterpret_cast<const ex_bf16x8*>(wr + i);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf(as[k * ff + i + e], static_cast<float>(wv[e]), s);
+          }
+          done = true;
+        }
+      }
+      if (!done)
+        for (int i = lane; i < ff; i += kWave) s = fmaf(as[k * ff + i], to_f32(wr[i]), s);
       total += weights[(size_t)t * top + k] * wave_sum(s);
     }
     if (lane == 0) y[(size_t)t * width + col] = from_f32<T>(total);

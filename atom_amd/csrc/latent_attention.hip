@@ -295,3 +295,118 @@ ATOM_EXPORT int atom_latent_attention(const void* q_abs, const void* pages, void
                                                  sink, heads, rank, rot, page_size, window));
   return launch_status();
 }
+
+// ------------------------------------------------------------------ the per-head products on the matrix cores
+//
+// The same product as heads_gemm with bfloat16 weights, for many rows: the head's weight rows are the A operand and
+// the tokens the B operand, both read straight from memory (a float32 input is rounded to bfloat16 on the way), so a
+// lane ends up with four consecutive columns of one token.  A block of 2 x 2 waves owns 64 tokens x 64 columns.
+// Needs k % 8 == 0 and offsets and strides of x that keep its 8-element pieces aligned.
+
+typedef __attribute__((ext_vector_type(4))) float hg_f32x4;
+typedef __attribute__((ext_vector_type(8))) __bf16 hg_bf16x8;
+
+__device__ __forceinline__ hg_bf16x8 hg_load8(const bf16_t* p, bool ok) {
+  const hg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? *reinterpret_cast<const hg_bf16x8*>(p) : zero;
+}
+
+__device__ __forceinline__ hg_bf16x8 hg_load8(const float* p, bool ok) {
+  hg_bf16x8 out = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (ok) {
+    const hg_f32x4 a = *reinterpret_cast<const hg_f32x4*>(p), b = *reinterpret_cast<const hg_f32x4*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[i] = static_cast<__bf16>(a[i]);
+      out[4 + i] = static_cast<__bf16>(b[i]);
+    }
+  }
+  return out;
+}
+
+template <typename TX, typename TY>
+__global__ void __launch_bounds__(256)
+heads_gemm_mfma_kernel(const TX* __restrict__ x, long ldx, long hsx, const bf16_t* __restrict__ w, TY* __restrict__ y,
+                       long ldy, long hsy, const float* __restrict__ gate, long ldg, int m, int n, int k, float alpha) {
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave, r = lane % 16, g = lane / 16;
+  const int h = blockIdx.z;
+  const int row0 = blockIdx.y * 64 + (wave / 2) * 32;
+  const int col0 = blockIdx.x * 64 + (wave % 2) * 32;
+  const TX* xrow[2];
+  bool rok[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int row = row0 + rt * 16 + r;
+    rok[rt] = row < m;
+    xrow[rt] = x + (size_t)(rok[rt] ? row : 0) * ldx + (size_t)h * hsx;
+  }
+  const bf16_t* wrow[2];
+  bool cok[2];
+#pragma unroll
+  for (int ct = 0; ct < 2; ++ct) {
+    const int col = col0 + ct * 16 + r;
+    cok[ct] = col < n;
+    wrow[ct] = w + ((size_t)h * n + (cok[ct] ? col : 0)) * k;
+  }
+  hg_f32x4 acc[2][2];
+#pragma unroll
+  for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) acc[ct][rt] = hg_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < k; k0 += 32) {
+    const int kk = k0 + 8 * g;
+    const bool kok = kk < k;
+    hg_bf16x8 xb[2], wa[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) xb[rt] = hg_load8(xrow[rt] + kk, kok && rok[rt]);
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) wa[ct] = hg_load8(wrow[ct] + kk, kok && cok[ct]);
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt)
+        acc[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ct], xb[rt], acc[ct][rt], 0, 0, 0);
+  }
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    const int row = row0 + rt * 16 + r;
+    if (row >= m) continue;
+    float f = alpha;
+    if (gate) f *= 1.f / (1.f + expf(-gate[(size_t)row * ldg + h]));
+#pragma unroll
+    for (int ct = 0; ct < 2; ++ct) {
+      const int col = col0 + ct * 16 + 4 * g;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (col + i < n) y[(size_t)row * ldy + (size_t)h * hsy + col + i] = from_f32<TY>(acc[ct][rt][i] * f);
+    }
+  }
+}
+
+ATOM_EXPORT int atom_heads_gemm_mfma_supports(int x_dtype, int w_dtype, long x_offset, long ldx, long hsx, int k) {
+  if (w_dtype != ATOM_BF16 || k % 8) return 0;
+  const long unit = x_dtype == ATOM_BF16 ? 8 : 4;   // elements of 16 bytes
+  return x_offset % unit == 0 && ldx % unit == 0 && hsx % unit == 0;
+}
+
+ATOM_EXPORT int atom_heads_gemm_mfma(const void* x, int x_dtype, long ldx, long hsx, const void* w, void* y, int y_dtype,
+                                     long ldy, long hsy, const float* gate, long ldg, int heads, int m, int n, int k,
+                                     float alpha, hipStream_t stream) {
+  if (m < 0 || n <= 0 || k <= 0 || heads <= 0 || heads > 65535 || (k % 8)) return ATOM_BAD_SHAPE;
+  if (x == nullptr || w == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
+  if ((unsigned)x_dtype > 1u || (unsigned)y_dtype > 1u) return ATOM_BAD_DTYPE;
+  if (m == 0) return ATOM_OK;
+  dim3 grid((n + 63) / 64, (m + 63) / 64, heads), block(256);
+  if (grid.y > 65535) return ATOM_TOO_LARGE;
+#define LAUNCH(TX, TY)                                                                                            \
+  hipLaunchKernelGGL((heads_gemm_mfma_kernel<TX, TY>), grid, block, 0, stream, (const TX*)x, ldx, hsx,           \
+                     (const bf16_t*)w, (TY*)y, ldy, hsy, gate, ldg, m, n, k, alpha)
+  switch (x_dtype * 2 + y_dtype) {
+    case 0: LAUNCH(float, float); break;
+    case 1: LAUNCH(float, bf16_t); break;
+    case 2: LAUNCH(bf16_t, float); break;
+    default: LAUNCH(bf16_t, bf16_t); break;
+  }
+#undef LAUNCH
+  return launch_status();
+}

@@ -245,21 +245,24 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
 __global__ void __launch_bounds__(128)
 latent_merge_kernel(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, const float* __restrict__ sink,
                     bf16_t* __restrict__ out, int heads, int rank, int parts) {
+  __shared__ float share[64];   // the parts' weights exp(m_p - M) / denominator
+  __shared__ float scratch[16];
   const size_t row = blockIdx.x;
   const int head = (int)(row % heads);
+  const int tid = threadIdx.x;
   const float* ml = ws_ml + row * parts * 2;
-  float top = sink ? sink[head] : -INFINITY;
-  for (int q = 0; q < parts; ++q) top = fmaxf(top, ml[2 * q]);
-  float denom = sink ? __expf(sink[head] - top) : 0.f;
-  if (top == -INFINITY) denom = 0.f;
-  for (int q = 0; q < parts; ++q)
-    if (ml[2 * q] != -INFINITY) denom += ml[2 * q + 1] * __expf(ml[2 * q] - top);
-  const float inv = denom > 0.f ? 1.f / denom : 0.f;
-  for (int e = threadIdx.x; e < rank; e += blockDim.x) {
+  const float sk = sink ? sink[head] : -INFINITY;
+  const float mine = tid < parts ? ml[2 * tid] : -INFINITY;
+  const float top = fmaxf(block_max(mine, scratch), sk);
+  const float w = (tid < parts && mine != -INFINITY) ? __expf(mine - top) : 0.f;
+  float denom = block_sum(tid < parts ? w * ml[2 * tid + 1] : 0.f, scratch);
+  if (sink && top != -INFINITY) denom += __expf(sk - top);
+  if (tid < parts) share[tid] = denom > 0.f ? w / denom : 0.f;
+  __syncthreads();
+  for (int e = tid; e < rank; e += 128) {
     float a = 0.f;
-    for (int q = 0; q < parts; ++q)
-      if (ml[2 * q] != -INFINITY) a += ws_o[(row * parts + q) * rank + e] * __expf(ml[2 * q] - top);
-    out[row * rank + e] = static_cast<bf16_t>(a * inv);
+    for (int q = 0; q < parts; ++q) a += ws_o[(row * parts + q) * rank + e] * share[q];
+    out[row * rank + e] = static_cast<bf16_t>(a);
   }
 }
 
@@ -312,7 +315,7 @@ ATOM_EXPORT int atom_latent_attention_mfma(const void* q, const void* pages, voi
   p.tpt = 64 / p.hpt;
   const int tiles = tokens / p.tpt + num_seqs;   // at least sum over requests of ceil(q_len / tpt)
   const int chunks = (heads + p.hpt - 1) / p.hpt;
-  if (chunks > 65535 || parts > 65535) return ATOM_TOO_LARGE;
+  if (chunks > 65535 || parts > 64) return ATOM_TOO_LARGE;   // the merge holds a weight per part in LDS
   const size_t smem = (size_t)kLChunk * latent_k_pitch(width) + (size_t)rank * kVPitch;
   if (smem > 160 * 1024) return ATOM_TOO_LARGE;
   dim3 grid(tiles, chunks, parts), block(256);

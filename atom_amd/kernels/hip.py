@@ -192,7 +192,8 @@ class HipKernels:
                    "atom_heads_gemm", "atom_latent_attention", "atom_conv_silu_state", "atom_delta_rule",
                    "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down",
                    "atom_latent_attention_mfma", "atom_latent_mfma_supports", "atom_latent_mfma_tokens_per_tile",
-                   "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports"):
+                   "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports",
+                   "atom_heads_gemm_mfma", "atom_heads_gemm_mfma_supports"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -220,6 +221,7 @@ class HipKernels:
         # routed experts: from this many (token, choice) pairs on, the pairs are sorted by expert and run as grouped
         # products on the matrix cores; below, every pair reads its expert's rows itself
         self.grouped_experts_from = 64
+        self.heads_mfma_from = 32      # rows from which the per-head products run on the matrix cores
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -922,8 +924,9 @@ class HipKernels:
         return out
 
     def linear_f32(self, x, weight, bias=None):
-        """``x @ weight.T (+ bias)`` by float32 multiply-adds whatever the operands' types, float32 out: for the
-        few products that have to be exact (a router's logits)."""
+        """``x @ weight.T (+ bias)`` summed in float32 whatever the operands' types, float32 out: for the few
+        products that have to be 32-bit sums (a router's logits).  bfloat16 operands take the engine's ordinary
+        products with float32 output; anything with a float32 operand runs plain float32 multiply-adds."""
         x = self.materialize(x)
         m, k = x.shape
         n = weight.shape[0]
@@ -931,6 +934,9 @@ class HipKernels:
         self._check("linear weight", weight, (torch.float32, torch.bfloat16), (n, k))
         if bias is not None:
             self._check("linear bias", bias, torch.float32, (n,))
+        if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and k % 8 == 0:
+            # products of two bfloat16 numbers are exact in float32, and the matrix cores add them in float32
+            return self.linear(x, weight, bias, out_dtype=torch.float32)
         y = torch.empty((m, n), dtype=torch.float32, device=x.device)
         self._done("gemm_f32", self.lib.atom_gemm_f32(_ptr(x), self._code(x), _ptr(weight), self._code(weight), _ptr(bias),
                                                       _ptr(y), F32, m, n, k, self._stream()))
@@ -983,6 +989,14 @@ class HipKernels:
             gp = ctypes.c_void_p(gate.data_ptr() + 4 * gate_offset)
         xp = ctypes.c_void_p(x.data_ptr() + x.element_size() * x_offset)
         yp = ctypes.c_void_p(y.data_ptr() + y.element_size() * y_offset)
+        if (weight.dtype == torch.bfloat16 and m >= self.heads_mfma_from and self.lib.atom_heads_gemm_mfma_supports(
+                self._code(x), BF16, ctypes.c_long(x_offset), ctypes.c_long(ldx), ctypes.c_long(hsx), k)):
+            # many rows: the same product on the matrix cores (a float32 input is rounded to bfloat16 on the way in)
+            self._done("heads_gemm_mfma", self.lib.atom_heads_gemm_mfma(
+                xp, self._code(x), ctypes.c_long(ldx), ctypes.c_long(hsx), _ptr(weight), yp, self._code(y),
+                ctypes.c_long(ldy), ctypes.c_long(hsy), gp, ctypes.c_long(ldg), heads, m, n, k, ctypes.c_float(alpha),
+                self._stream()))
+            return y
         self._done("heads_gemm", self.lib.atom_heads_gemm(
             xp, self._code(x), ctypes.c_long(ldx), ctypes.c_long(hsx), _ptr(weight), self._code(weight), yp,
             self._code(y), ctypes.c_long(ldy), ctypes.c_long(hsy), gp, ctypes.c_long(ldg), heads, m, n, k,

@@ -134,6 +134,24 @@ def test_latent_prepare(dtype, heads, dim, rot, rank, dims, scaling):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("x_dtype", DTYPES)
+@pytest.mark.parametrize("H,m,n,k", [(3, 70, 21, 16), (2, 200, 100, 40), (5, 33, 64, 128)])
+def test_heads_gemm_on_the_matrix_cores(dtype, x_dtype, H, m, n, k):
+    """Strides that keep 16-byte pieces aligned: bfloat16 weights with 32 rows or more take the matrix-core kernel."""
+    ops = gpu_ops()
+    ldx, hsx, ldy, hsy = H * (k + 8) + 16, k + 8, H * (n + 3), n + 3
+    x = rnd((m, ldx), 1).to(x_dtype)
+    w = rnd((H, n, k), 2, k ** -0.5).to(dtype)
+    y = torch.zeros((m, ldy), dtype=dtype, device=DEV)
+    gate = rnd((m, H + 2), 3)
+    ops.heads_gemm(x.to(DEV), 8, ldx, hsx, w.to(DEV), y, 1, ldy, hsy, H, m, n, k, alpha=0.7, gate=gate.to(DEV),
+                   gate_offset=2, ldg=H + 2)
+    for h in range(H):
+        want = 0.7 * x.double()[:, 8 + h * hsx:8 + h * hsx + k] @ w.double()[h].T * torch.sigmoid(gate.double()[:, 2 + h])[:, None]
+        close(y[:, 1 + h * hsy:1 + h * hsy + n], want, torch.bfloat16 if torch.bfloat16 in (dtype, x_dtype) else dtype, f"head {h}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_heads_gemm_with_strides_and_gate(dtype):
     ops = gpu_ops()
     H, m, n, k = 3, 70, 21, 13
