@@ -10,7 +10,7 @@
 // Requests are walked through the step's device arrays (cu_seqlens_q, slot_of_seq), so the same kernels serve
 // prompt portions, single tokens and padded rows (slot < 0: nothing is read or written) of a replayed graph.
 //
-//   conv_silu_state   one thread per (request, channel) walks the request's tokens of this step
+//   conv_silu_state   one thread per (request, channel, run of 64 tokens)
 //   delta_rule        blocks per (request, head, group of columns); a column of S (over dim) sits in the registers of up
 //                     to 16 adjacent lanes, so the columns never meet; q, k and the gates of a run of tokens are
 //                     staged in LDS
@@ -19,6 +19,10 @@
 
 constexpr int kMaxTaps = 8;
 
+constexpr int kConvRun = 64;   // tokens of a request that one block takes
+
+// grid (channel blocks, requests, runs of 64 tokens).  Only a request's first run reads the carried inputs, and it
+// alone writes them back (after its reads), so the runs never meet.
 template <typename TW>
 __global__ void __launch_bounds__(256)
 conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restrict__ taps_w, int taps, int channels,
@@ -28,9 +32,12 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
   const int seq = blockIdx.y;
   if (c >= channels) return;
   const int begin = cu_seqlens[seq], end = cu_seqlens[seq + 1];
+  const int first = begin + blockIdx.z * kConvRun;
+  if (first >= end && !(blockIdx.z == 0)) return;
+  const int last = first + kConvRun < end ? first + kConvRun : end;
   const int slot = slot_of_seq[seq];
   if (slot < 0) {
-    for (int t = begin; t < end; ++t) y[(size_t)t * channels + c] = 0.f;
+    for (int t = first; t < last; ++t) y[(size_t)t * channels + c] = 0.f;
     return;
   }
   float w[kMaxTaps], win[kMaxTaps];   // win[taps - 1] is the current input
@@ -39,11 +46,16 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
     w[j] = j < taps ? to_f32(taps_w[(size_t)c * taps + j]) : 0.f;
     win[j] = 0.f;
   }
-  float* tail = state + (size_t)slot * slot_stride;   // [taps - 1, channels]
+  float* tail = state + (size_t)slot * slot_stride;   // [taps - 1, channels], oldest first
+  // the taps - 1 inputs before `first`: the step's own tokens where there are enough, else the carried ones
 #pragma unroll
-  for (int j = 0; j < kMaxTaps - 1; ++j)
-    if (j < taps - 1) win[j + 1] = tail[(size_t)j * channels + c];   // shifted down by the first token below
-  for (int t = begin; t < end; ++t) {
+  for (int j = 0; j < kMaxTaps - 1; ++j) {
+    if (j < taps - 1) {
+      const int t = first - (taps - 1) + j;   // the token whose input this is
+      win[j + 1] = t >= begin ? x[(size_t)t * ldx + c] : tail[(size_t)(j + (first - begin)) * channels + c];
+    }
+  }
+  for (int t = first; t < last; ++t) {
 #pragma unroll
     for (int j = 0; j < kMaxTaps - 1; ++j) win[j] = win[j + 1];
     const float cur = x[(size_t)t * ldx + c];
@@ -56,20 +68,35 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
       if (j < taps) s = fmaf(w[j], win[j], s);
     y[(size_t)t * channels + c] = s / (1.f + expf(-s));
   }
+  if (blockIdx.z == 0) {
+    // the request's last taps - 1 inputs after this step
+    const int n = end - begin;
 #pragma unroll
-  for (int j = 0; j < kMaxTaps - 1; ++j)
-    if (j < taps - 1) tail[(size_t)j * channels + c] = win[j + 1];
+    for (int j = 0; j < kMaxTaps - 1; ++j) {
+      if (j < taps - 1) {
+        const int back = taps - 1 - j;          // this entry is the input `back` tokens before the next one
+        float v;
+        if (back <= n) v = x[(size_t)(end - back) * ldx + c];
+        else v = tail[(size_t)(j + n) * channels + c];   // still one of the carried ones, moved up by n
+        win[j] = v;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kMaxTaps - 1; ++j)
+      if (j < taps - 1) tail[(size_t)j * channels + c] = win[j];
+  }
 }
 
 ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w, int w_dtype, int taps, int channels,
                                      float* state, long slot_stride, const int* cu_seqlens, const int* slot_of_seq,
-                                     int num_seqs, float* y, hipStream_t stream) {
+                                     int num_seqs, int max_q_len, float* y, hipStream_t stream) {
   if (taps < 1 || taps > kMaxTaps) return ATOM_TOO_LARGE;
   if (channels <= 0 || ldx < channels || num_seqs < 0 || slot_stride < (long)(taps - 1) * channels) return ATOM_BAD_SHAPE;
-  if (x == nullptr || taps_w == nullptr || state == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
+  if (x == nullptr || taps_w == nullptr || state == nullptr || y == nullptr || max_q_len < 0) return ATOM_BAD_SHAPE;
   if (num_seqs == 0) return ATOM_OK;
-  if (num_seqs > 65535) return ATOM_TOO_LARGE;
-  dim3 grid((channels + 255) / 256, num_seqs), block(256);
+  const int runs = max_q_len > 0 ? (max_q_len + kConvRun - 1) / kConvRun : 1;
+  if (num_seqs > 65535 || runs > 65535) return ATOM_TOO_LARGE;
+  dim3 grid((channels + 255) / 256, num_seqs, runs), block(256);
   ATOM_DISPATCH_DTYPE(w_dtype, hipLaunchKernelGGL((conv_silu_state_kernel<T>), grid, block, 0, stream, x, ldx,
                                                    (const T*)taps_w, taps, channels, state, slot_stride, cu_seqlens,
                                                    slot_of_seq, y));
@@ -77,6 +104,23 @@ ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w
 }
 
 // ------------------------------------------------------------------ the recurrence
+
+// The sum of v over the LPC adjacent lanes that share a column, in each of them, through the data-parallel
+// permutes of one row of 16 lanes (no trip through LDS): neighbours, pairs, then the mirrored half-row and row,
+// which hold the same sums as the lanes they stand for once the smaller groups are summed.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+template <int LPC>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (LPC >= 2) v = dpp_add<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if constexpr (LPC >= 4) v = dpp_add<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if constexpr (LPC >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if constexpr (LPC >= 16) v = dpp_add<0x140>(v);  // row_mirror
+  return v;
+}
 
 constexpr int kRun = 16;   // tokens whose q, k and gates are staged at once
 constexpr int kDPL = 16;   // entries of a column of S that one lane holds
@@ -152,9 +196,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
         S[e] *= g;
         part[e & 3] = fmaf(S[e], ks[j][e * LPC + sub], part[e & 3]);
       }
-      float dot = (part[0] + part[1]) + (part[2] + part[3]);
-#pragma unroll
-      for (int off = 1; off < LPC; off <<= 1) dot += __shfl_xor(dot, off, kWave);
+      const float dot = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
       const float u = beta * (v - dot);
       part[0] = part[1] = part[2] = part[3] = 0.f;
 #pragma unroll
@@ -162,9 +204,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
         S[e] = fmaf(ks[j][e * LPC + sub], u, S[e]);
         part[e & 3] = fmaf(S[e], qs[j][e * LPC + sub], part[e & 3]);
       }
-      float o = (part[0] + part[1]) + (part[2] + part[3]);
-#pragma unroll
-      for (int off = 1; off < LPC; off <<= 1) o += __shfl_xor(o, off, kWave);
+      const float o = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
       if (live && sub == 0) out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
     }
   }

@@ -43,11 +43,70 @@ __global__ void router_choose_kernel(const float* __restrict__ logits, const flo
     for (int k = 0; k < top; ++k) w[k] /= total;
 }
 
+// A wave per token: lane l holds the scores of experts l, l + 64, ... (up to 8 of them, so up to 512 experts); each
+// of the `top` rounds is a maximum over the wave of (choice score, lower index first).
+constexpr int kRouterPerLane = 8;
+
+__global__ void __launch_bounds__(256)
+router_choose_wave_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
+                          int* __restrict__ ids, float* __restrict__ weights, int tokens, int experts, int top,
+                          int renormalize) {
+  const int t = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (t >= tokens) return;
+  const int lane = threadIdx.x % kWave;
+  float score[kRouterPerLane], plain[kRouterPerLane];
+#pragma unroll
+  for (int j = 0; j < kRouterPerLane; ++j) {
+    const int e = lane + j * kWave;
+    if (e < experts) {
+      plain[j] = 1.f / (1.f + expf(-logits[(size_t)t * experts + e]));
+      score[j] = plain[j] + (correction ? correction[e] : 0.f);
+    } else {
+      plain[j] = 0.f;
+      score[j] = -INFINITY;
+    }
+  }
+  float total = 0.f, mine = 0.f;   // lane k keeps the weight of choice k (top <= 64)
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY, best_plain = 0.f;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; ++j)
+      if (score[j] > best) {
+        best = score[j];
+        best_plain = plain[j];
+        best_e = lane + j * kWave;
+      }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, kWave), op = __shfl_xor(best_plain, off, kWave);
+      const int oe = __shfl_xor(best_e, off, kWave);
+      if (ob > best || (ob == best && oe < best_e)) {
+        best = ob;
+        best_plain = op;
+        best_e = oe;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; ++j)
+      if (lane + j * kWave == best_e) score[j] = -INFINITY;
+    if (lane == 0) ids[(size_t)t * top + k] = best_e;
+    if (lane == k) mine = best_plain;
+    total += best_plain;
+  }
+  if (lane < top) weights[(size_t)t * top + lane] = renormalize ? mine / total : mine;
+}
+
 ATOM_EXPORT int atom_router_choose(const float* logits, const float* correction, int* ids, float* weights, int tokens,
                                    int experts, int top, int renormalize, hipStream_t stream) {
   if (tokens < 0 || experts <= 0 || top <= 0 || top > experts) return ATOM_BAD_SHAPE;
   if (logits == nullptr || ids == nullptr || weights == nullptr) return ATOM_BAD_SHAPE;
   if (tokens == 0) return ATOM_OK;
+  if (experts <= kRouterPerLane * kWave && top <= kWave) {
+    hipLaunchKernelGGL(router_choose_wave_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, logits, correction, ids,
+                       weights, tokens, experts, top, renormalize);
+    return launch_status();
+  }
   hipLaunchKernelGGL(router_choose_kernel, dim3((tokens + 127) / 128), dim3(128), 0, stream, logits, correction, ids,
                      weights, tokens, experts, top, renormalize);
   return launch_status();

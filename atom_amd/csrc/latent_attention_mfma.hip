@@ -123,35 +123,60 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
   const int groups = p.width / 8;
   const int keyA0 = 8 * (r / 4) + (r % 4);   // the key of A row r in the first score tile; the second: + 4
 
-  for (int c = my_lo; c < my_hi; ++c) {
+  // a chunk's rows travel memory -> registers -> LDS; the registers are filled for the next chunk while this one
+  // is multiplied, so that the memory's latency is hidden behind the products
+  constexpr int ITEMS = (KS * 64 + 255) / 256;   // (pair of keys, 8 entries) items a thread moves, at most
+  bf16x8 ra[ITEMS], rb[ITEMS];
+  auto fetch = [&](int c) {
     const int kbase = c * kLChunk;
-    __syncthreads();   // the chunk before has been read
-    for (int item = tid; item < (kLChunk / 2) * groups; item += 256) {
-      const int kp = item / groups, dg = item - kp * groups;
-      const int key0 = kbase + 2 * kp;
-      bf16x8 a = zero8, b2 = zero8;
-      if (key0 <= last_pos) {
-        const size_t row = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
-        a = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
-      }
-      if (key0 + 1 <= last_pos) {
-        const size_t row = (size_t)table[(key0 + 1) / p.page_size] * p.page_size + (key0 + 1) % p.page_size;
-        b2 = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
-      }
-      *reinterpret_cast<bf16x8*>(klds + (2 * kp) * kpitch + dg * 16) = a;
-      *reinterpret_cast<bf16x8*>(klds + (2 * kp + 1) * kpitch + dg * 16) = b2;
-      if (dg * 8 < p.rank) {
-        // entry i of both keys side by side: the halves of the rows' 32-bit words
-        const u32x4 wa = __builtin_bit_cast(u32x4, a), wb = __builtin_bit_cast(u32x4, b2);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const unsigned lo16 = (i & 1) ? wa[i / 2] >> 16 : wa[i / 2] & 0xffffu;
-          const unsigned hi16 = (i & 1) ? wb[i / 2] >> 16 : wb[i / 2] & 0xffffu;
-          *reinterpret_cast<unsigned*>(vlds + (dg * 8 + i) * kVPitch + kp * 4) = lo16 | (hi16 << 16);
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * 256;
+      ra[it] = zero8;
+      rb[it] = zero8;
+      if (item < (kLChunk / 2) * groups) {
+        const int kp = item / groups, dg = item - kp * groups;
+        const int key0 = kbase + 2 * kp;
+        if (key0 <= last_pos) {
+          const size_t row = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
+          ra[it] = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
+        }
+        if (key0 + 1 <= last_pos) {
+          const size_t row = (size_t)table[(key0 + 1) / p.page_size] * p.page_size + (key0 + 1) % p.page_size;
+          rb[it] = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
         }
       }
     }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * 256;
+      if (item < (kLChunk / 2) * groups) {
+        const int kp = item / groups, dg = item - kp * groups;
+        *reinterpret_cast<bf16x8*>(klds + (2 * kp) * kpitch + dg * 16) = ra[it];
+        *reinterpret_cast<bf16x8*>(klds + (2 * kp + 1) * kpitch + dg * 16) = rb[it];
+        if (dg * 8 < p.rank) {
+          // entry i of both keys side by side: the halves of the rows' 32-bit words
+          const u32x4 wa = __builtin_bit_cast(u32x4, ra[it]), wb = __builtin_bit_cast(u32x4, rb[it]);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const unsigned lo16 = (i & 1) ? wa[i / 2] >> 16 : wa[i / 2] & 0xffffu;
+            const unsigned hi16 = (i & 1) ? wb[i / 2] >> 16 : wb[i / 2] & 0xffffu;
+            *reinterpret_cast<unsigned*>(vlds + (dg * 8 + i) * kVPitch + kp * 4) = lo16 | (hi16 << 16);
+          }
+        }
+      }
+    }
+  };
+  if (my_lo < my_hi) fetch(my_lo);
+
+  for (int c = my_lo; c < my_hi; ++c) {
+    const int kbase = c * kLChunk;
+    __syncthreads();   // the chunk before has been read
+    stash();
     __syncthreads();
+    if (c + 1 < my_hi) fetch(c + 1);
     if (!wave_busy) continue;
 
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};

@@ -221,7 +221,7 @@ class HipKernels:
         # routed experts: from this many (token, choice) pairs on, the pairs are sorted by expert and run as grouped
         # products on the matrix cores; below, every pair reads its expert's rows itself
         self.grouped_experts_from = 64
-        self.heads_mfma_from = 32      # rows from which the per-head products run on the matrix cores
+        self.heads_mfma_from = 1       # rows from which the per-head products run on the matrix cores
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -1056,11 +1056,13 @@ class HipKernels:
 
     # ------------------------------------------------------------------ the gated delta rule
 
-    def conv_silu_state(self, x, channels: int, taps_weight, state, cu_seqlens_q, slot_of_seq, out):
+    def conv_silu_state(self, x, channels: int, taps_weight, state, cu_seqlens_q, slot_of_seq, out,
+                        max_q_len: int | None = None):
         """Short causal convolution per channel over each request's tokens, then SiLU.  ``x`` float32 [tokens, >=
         channels] (the first ``channels`` columns are convolved); ``taps_weight`` [channels, taps], last column the
         current token's; ``state`` float32 [slots, >= (taps - 1) * channels]: a request's last taps - 1 inputs, read
-        and written back.  Requests with slot -1 are padding."""
+        and written back.  Requests with slot -1 are padding.  ``max_q_len``: the most tokens a request brings (an
+        upper bound sizes the grid; default: all tokens)."""
         tokens, ldx = x.shape
         taps = taps_weight.shape[1]
         seqs = slot_of_seq.numel()
@@ -1072,7 +1074,8 @@ class HipKernels:
         self._check("convolution out", out, torch.float32, (tokens, channels))
         self._done("conv_silu_state", self.lib.atom_conv_silu_state(
             _ptr(x), ldx, _ptr(taps_weight), self._code(taps_weight), taps, channels, _ptr(state),
-            ctypes.c_long(state.shape[1]), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs, _ptr(out), self._stream()))
+            ctypes.c_long(state.shape[1]), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
+            tokens if max_q_len is None else min(tokens, max_q_len), _ptr(out), self._stream()))
         return out
 
     def delta_rule(self, qkv, gates, a_off: int, b_off: int, a_log, dt_bias, state, state_off: int, cu_seqlens_q,

@@ -69,7 +69,8 @@ class GatedDeltaRule(Mixer):
         H, dv, C = self.num_heads, self.value_dim, self.channels
         proj = ops.linear(x, self.params["proj.weight"], None, out_dtype=torch.float32)
         qkv = torch.empty((T, C), dtype=torch.float32, device=x.device)
-        ops.conv_silu_state(proj, C, self.params["conv.weight"], cache.state, ctx.cu_seqlens_q, ctx.slot_of_seq, qkv)
+        ops.conv_silu_state(proj, C, self.params["conv.weight"], cache.state, ctx.cu_seqlens_q, ctx.slot_of_seq, qkv,
+                            max_q_len=ctx.max_q_len)
         read = torch.empty((T, H, dv), dtype=torch.float32, device=x.device)
         gate_off = C
         beta_off = C + H * dv

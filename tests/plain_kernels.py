@@ -213,7 +213,7 @@ class PlainKernels:
             out[t] = ((e / denom) @ rows[:, :rank]).to(out.dtype)
         return out
 
-    def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out):
+    def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out, max_q_len=None):
         taps = taps_weight.shape[1]
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
