@@ -187,9 +187,16 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       bs[tid] = 1.f / (1.f + expf(-r[b_off + head]));
     }
     __syncthreads();
-    for (int j = 0; j < n; ++j) {
+    // the run's values of this column, asked for at once: a load inside the chain below would be waited for
+    float vv[kRun];
+#pragma unroll
+    for (int j = 0; j < kRun; ++j)
+      vv[j] = (live && j < n) ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+#pragma unroll
+    for (int j = 0; j < kRun; ++j) {
+      if (j >= n) break;
       const float g = gs[j], beta = bs[j];
-      const float v = live ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+      const float v = vv[j];
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int e = 0; e < kDPL; ++e) {

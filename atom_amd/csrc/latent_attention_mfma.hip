@@ -124,7 +124,9 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
   const int keyA0 = 8 * (r / 4) + (r % 4);   // the key of A row r in the first score tile; the second: + 4
 
   // a chunk's rows travel memory -> registers -> LDS; the registers are filled for the next chunk while this one
-  // is multiplied, so that the memory's latency is hidden behind the products
+  // is multiplied, so that the memory's latency is hidden behind the products.  Work is dealt out with the pair of
+  // keys running fastest: 16 lanes then write 16 consecutive words of a transposed row (consecutive banks), and
+  // four such groups of lanes read one whole 64-byte line of each of their 32 rows.
   constexpr int ITEMS = (KS * 64 + 255) / 256;   // (pair of keys, 8 entries) items a thread moves, at most
   bf16x8 ra[ITEMS], rb[ITEMS];
   auto fetch = [&](int c) {
@@ -135,7 +137,7 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
       ra[it] = zero8;
       rb[it] = zero8;
       if (item < (kLChunk / 2) * groups) {
-        const int kp = item / groups, dg = item - kp * groups;
+        const int kp = item % (kLChunk / 2), dg = item / (kLChunk / 2);
         const int key0 = kbase + 2 * kp;
         if (key0 <= last_pos) {
           const size_t row = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
@@ -153,7 +155,7 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
     for (int it = 0; it < ITEMS; ++it) {
       const int item = tid + it * 256;
       if (item < (kLChunk / 2) * groups) {
-        const int kp = item / groups, dg = item - kp * groups;
+        const int kp = item % (kLChunk / 2), dg = item / (kLChunk / 2);
         *reinterpret_cast<bf16x8*>(klds + (2 * kp) * kpitch + dg * 16) = ra[it];
         *reinterpret_cast<bf16x8*>(klds + (2 * kp + 1) * kpitch + dg * 16) = rb[it];
         if (dg * 8 < p.rank) {
