@@ -168,16 +168,23 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   for (int t0 = begin; t0 < end; t0 += kRun) {
     const int n = end - t0 < kRun ? end - t0 : kRun;
     __syncthreads();   // the previous run's q and k have been read
-    // unit vectors: a wave per (token, q or k)
+    // the run's q and k rows: every thread asks for its share at once, then a wave per (token, q or k) makes the
+    // row a unit vector in place
+    for (int idx = tid; idx < 2 * n * DMAX; idx += 256) {
+      const int item = idx / DMAX, i = idx - item * DMAX;
+      const int j = item >> 1, is_k = item & 1;
+      const float v = i < dim ? qkv[(size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim + i] : 0.f;
+      (is_k ? ks[j] : qs[j])[i] = v;
+    }
+    __syncthreads();
     for (int item = wave; item < 2 * n; item += 4) {
       const int j = item >> 1, is_k = item & 1;
-      const float* src = qkv + (size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim;
+      float* dst = is_k ? ks[j] : qs[j];
       float ss = 0.f;
-      for (int i = lane; i < dim; i += kWave) ss += src[i] * src[i];
+      for (int i = lane; i < DMAX; i += kWave) ss += dst[i] * dst[i];
       ss = wave_sum(ss);
       const float f = (is_k ? 1.f : q_scale) / sqrtf(ss + 1e-6f);
-      float* dst = is_k ? ks[j] : qs[j];
-      for (int i = lane; i < DMAX; i += kWave) dst[i] = i < dim ? src[i] * f : 0.f;
+      for (int i = lane; i < DMAX; i += kWave) dst[i] *= f;
     }
     if (tid < n) {
       const float* r = ab + (size_t)(t0 + tid) * ld_ab;

@@ -129,38 +129,43 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
   // four such groups of lanes read one whole 64-byte line of each of their 32 rows.
   constexpr int ITEMS = (KS * 64 + 255) / 256;   // (pair of keys, 8 entries) items a thread moves, at most
   bf16x8 ra[ITEMS], rb[ITEMS];
+  // without a branch: every lookup and every row load of a chunk is asked for before any is waited for.  Keys
+  // beyond the last visible one are read as that one and replaced by zeros when they are staged.
+  const int n_items = (kLChunk / 2) * groups;
   auto fetch = [&](int c) {
+    const int kbase = c * kLChunk;
+    size_t row_a[ITEMS], row_b[ITEMS];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * 256 < n_items ? tid + it * 256 : n_items - 1;
+      const int kp = item % (kLChunk / 2);
+      const int key0 = kbase + 2 * kp < last_pos ? kbase + 2 * kp : last_pos;
+      const int key1 = key0 + 1 < last_pos ? key0 + 1 : last_pos;
+      row_a[it] = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
+      row_b[it] = (size_t)table[key1 / p.page_size] * p.page_size + key1 % p.page_size;
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int item = tid + it * 256 < n_items ? tid + it * 256 : n_items - 1;
+      const int dg = item / (kLChunk / 2);
+      ra[it] = *reinterpret_cast<const bf16x8*>(p.pages + row_a[it] * p.width + dg * 8);
+      rb[it] = *reinterpret_cast<const bf16x8*>(p.pages + row_b[it] * p.width + dg * 8);
+    }
+  };
+  auto stash = [&](int c) {
     const int kbase = c * kLChunk;
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
       const int item = tid + it * 256;
-      ra[it] = zero8;
-      rb[it] = zero8;
-      if (item < (kLChunk / 2) * groups) {
+      if (item < n_items) {
         const int kp = item % (kLChunk / 2), dg = item / (kLChunk / 2);
-        const int key0 = kbase + 2 * kp;
-        if (key0 <= last_pos) {
-          const size_t row = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
-          ra[it] = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
-        }
-        if (key0 + 1 <= last_pos) {
-          const size_t row = (size_t)table[(key0 + 1) / p.page_size] * p.page_size + (key0 + 1) % p.page_size;
-          rb[it] = *reinterpret_cast<const bf16x8*>(p.pages + row * p.width + dg * 8);
-        }
-      }
-    }
-  };
-  auto stash = [&]() {
-#pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      const int item = tid + it * 256;
-      if (item < (kLChunk / 2) * groups) {
-        const int kp = item % (kLChunk / 2), dg = item / (kLChunk / 2);
-        *reinterpret_cast<bf16x8*>(klds + (2 * kp) * kpitch + dg * 16) = ra[it];
-        *reinterpret_cast<bf16x8*>(klds + (2 * kp + 1) * kpitch + dg * 16) = rb[it];
+        const bf16x8 va = kbase + 2 * kp <= last_pos ? ra[it] : zero8;
+        const bf16x8 vb = kbase + 2 * kp + 1 <= last_pos ? rb[it] : zero8;
+        *reinterpret_cast<bf16x8*>(klds + (2 * kp) * kpitch + dg * 16) = va;
+        *reinterpret_cast<bf16x8*>(klds + (2 * kp + 1) * kpitch + dg * 16) = vb;
         if (dg * 8 < p.rank) {
           // entry i of both keys side by side: the halves of the rows' 32-bit words
-          const u32x4 wa = __builtin_bit_cast(u32x4, ra[it]), wb = __builtin_bit_cast(u32x4, rb[it]);
+          const u32x4 wa = __builtin_bit_cast(u32x4, va), wb = __builtin_bit_cast(u32x4, vb);
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
             const unsigned lo16 = (i & 1) ? wa[i / 2] >> 16 : wa[i / 2] & 0xffffu;
@@ -176,7 +181,7 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
   for (int c = my_lo; c < my_hi; ++c) {
     const int kbase = c * kLChunk;
     __syncthreads();   // the chunk before has been read
-    stash();
+    stash(c);
     __syncthreads();
     if (c + 1 < my_hi) fetch(c + 1);
     if (!wave_busy) continue;
