@@ -165,18 +165,50 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   const float q_scale = 1.f / sqrtf((float)dim);
   const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
   const int wave = tid / kWave, lane = tid % kWave;
+  // A run's q and k rows, its values of this column and its gates travel memory -> registers -> LDS; the registers
+  // are filled for the next run while this run's tokens are worked through, so that no load is waited for inside
+  // the chain of tokens.
+  constexpr int QK_ITEMS = 2 * kRun * DMAX / 256;
+  float qk_raw[QK_ITEMS], v_next[kRun], a_next = 0.f, b_next = 0.f;
+  auto load_run = [&](int t0) {
+    const int n = end - t0 < kRun ? end - t0 : kRun;
+#pragma unroll
+    for (int it = 0; it < QK_ITEMS; ++it) {
+      const int idx = tid + it * 256;
+      const int item = idx / DMAX, i = idx % DMAX;
+      const int j = item >> 1, is_k = item & 1;
+      qk_raw[it] = (j < n && i < dim) ? qkv[(size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim + i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kRun; ++j)
+      v_next[j] = (live && j < n) ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+    if (tid < n) {
+      const float* r = ab + (size_t)(t0 + tid) * ld_ab;
+      a_next = r[a_off + head];
+      b_next = r[b_off + head];
+    }
+  };
+  if (begin < end) load_run(begin);
   for (int t0 = begin; t0 < end; t0 += kRun) {
     const int n = end - t0 < kRun ? end - t0 : kRun;
     __syncthreads();   // the previous run's q and k have been read
-    // the run's q and k rows: every thread asks for its share at once, then a wave per (token, q or k) makes the
-    // row a unit vector in place
-    for (int idx = tid; idx < 2 * n * DMAX; idx += 256) {
-      const int item = idx / DMAX, i = idx - item * DMAX;
-      const int j = item >> 1, is_k = item & 1;
-      const float v = i < dim ? qkv[(size_t)(t0 + j) * channels + (is_k ? k_off : 0) + kvh * dim + i] : 0.f;
-      (is_k ? ks[j] : qs[j])[i] = v;
+#pragma unroll
+    for (int it = 0; it < QK_ITEMS; ++it) {
+      const int idx = tid + it * 256;
+      const int item = idx / DMAX, i = idx % DMAX;
+      ((item & 1) ? ks[item >> 1] : qs[item >> 1])[i] = qk_raw[it];
     }
+    if (tid < n) {
+      const float z = a_next + bias;
+      const float sp_z = z > 20.f ? z : log1pf(expf(z));
+      gs[tid] = expf(decay_rate * sp_z);
+      bs[tid] = 1.f / (1.f + expf(-b_next));
+    }
+    float vv[kRun];
+#pragma unroll
+    for (int j = 0; j < kRun; ++j) vv[j] = v_next[j];
     __syncthreads();
+    // unit vectors: a wave per (token, q or k), in place
     for (int item = wave; item < 2 * n; item += 4) {
       const int j = item >> 1, is_k = item & 1;
       float* dst = is_k ? ks[j] : qs[j];
@@ -186,19 +218,8 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       const float f = (is_k ? 1.f : q_scale) / sqrtf(ss + 1e-6f);
       for (int i = lane; i < DMAX; i += kWave) dst[i] *= f;
     }
-    if (tid < n) {
-      const float* r = ab + (size_t)(t0 + tid) * ld_ab;
-      const float z = r[a_off + head] + bias;
-      const float sp_z = z > 20.f ? z : log1pf(expf(z));
-      gs[tid] = expf(decay_rate * sp_z);
-      bs[tid] = 1.f / (1.f + expf(-r[b_off + head]));
-    }
     __syncthreads();
-    // the run's values of this column, asked for at once: a load inside the chain below would be waited for
-    float vv[kRun];
-#pragma unroll
-    for (int j = 0; j < kRun; ++j)
-      vv[j] = (live && j < n) ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+    if (t0 + kRun < end) load_run(t0 + kRun);
 #pragma unroll
     for (int j = 0; j < kRun; ++j) {
       if (j >= n) break;

@@ -36,6 +36,7 @@ struct LatentParams {
   const int* block_tables;  // [num_seqs, max_blocks]
   const float* sink;        // [heads] or null
   int num_seqs, max_blocks, heads, rank, width, page_size, window, parts, hpt, tpt;
+  int page_shift;           // log2(page_size) where that is a power of two of at least 8, else -1
 };
 
 constexpr int kLChunk = 32;
@@ -135,14 +136,36 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
   auto fetch = [&](int c) {
     const int kbase = c * kLChunk;
     size_t row_a[ITEMS], row_b[ITEMS];
+    if (p.page_shift >= 0) {
+      // pages of 8, 16, 32, ... keys: a chunk lies in at most four pages, whose numbers every lane needs alike
+      // (uniform loads), and places within a page are shifts and masks
+      const int pbase = kbase >> p.page_shift, plast = last_pos >> p.page_shift;
+      int tab[4];
 #pragma unroll
-    for (int it = 0; it < ITEMS; ++it) {
-      const int item = tid + it * 256 < n_items ? tid + it * 256 : n_items - 1;
-      const int kp = item % (kLChunk / 2);
-      const int key0 = kbase + 2 * kp < last_pos ? kbase + 2 * kp : last_pos;
-      const int key1 = key0 + 1 < last_pos ? key0 + 1 : last_pos;
-      row_a[it] = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
-      row_b[it] = (size_t)table[key1 / p.page_size] * p.page_size + key1 % p.page_size;
+      for (int j = 0; j < 4; ++j) tab[j] = table[pbase + j < plast ? pbase + j : plast];
+      const int mask = p.page_size - 1;
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int item = tid + it * 256 < n_items ? tid + it * 256 : n_items - 1;
+        const int kp = item % (kLChunk / 2);
+        const int key0 = kbase + 2 * kp < last_pos ? kbase + 2 * kp : last_pos;
+        const int key1 = key0 + 1 < last_pos ? key0 + 1 : last_pos;
+        const int j0 = (key0 >> p.page_shift) - pbase, j1 = (key1 >> p.page_shift) - pbase;
+        const int page0 = j0 == 0 ? tab[0] : j0 == 1 ? tab[1] : j0 == 2 ? tab[2] : tab[3];
+        const int page1 = j1 == 0 ? tab[0] : j1 == 1 ? tab[1] : j1 == 2 ? tab[2] : tab[3];
+        row_a[it] = ((size_t)page0 << p.page_shift) | (size_t)(key0 & mask);
+        row_b[it] = ((size_t)page1 << p.page_shift) | (size_t)(key1 & mask);
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int item = tid + it * 256 < n_items ? tid + it * 256 : n_items - 1;
+        const int kp = item % (kLChunk / 2);
+        const int key0 = kbase + 2 * kp < last_pos ? kbase + 2 * kp : last_pos;
+        const int key1 = key0 + 1 < last_pos ? key0 + 1 : last_pos;
+        row_a[it] = (size_t)table[key0 / p.page_size] * p.page_size + key0 % p.page_size;
+        row_b[it] = (size_t)table[key1 / p.page_size] * p.page_size + key1 % p.page_size;
+      }
     }
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
@@ -345,6 +368,9 @@ ATOM_EXPORT int atom_latent_attention_mfma(const void* q, const void* pages, voi
   p.parts = parts;
   p.hpt = heads < 64 ? heads : 64;
   p.tpt = 64 / p.hpt;
+  p.page_shift = -1;
+  for (int sh = 3; sh < 20; ++sh)
+    if (page_size == (1 << sh)) p.page_shift = sh;
   const int tiles = tokens / p.tpt + num_seqs;   // at least sum over requests of ceil(q_len / tpt)
   const int chunks = (heads + p.hpt - 1) / p.hpt;
   if (chunks > 65535 || parts > 64) return ATOM_TOO_LARGE;   // the merge holds a weight per part in LDS

@@ -267,10 +267,12 @@ def test_latent_attention_single_tokens_with_keys_split_over_blocks(dtype, rank,
 # ------------------------------------------------------------------ the delta rule
 
 
+@pytest.mark.parametrize("lens", [[5, 1, 2, 1, 9], [150, 3, 64, 2, 65]])
 @pytest.mark.parametrize("taps,channels", [(2, 40), (4, 300), (5, 17), (1, 8)])
-def test_conv_silu_state(taps, channels):
+def test_conv_silu_state(taps, channels, lens):
+    """Requests of one token, of fewer tokens than taps, and of several runs of 64 tokens; a padding row."""
     ops = gpu_ops()
-    lens, slots = [5, 1, 2, 1, 9], [2, 0, 3, -1, 1]
+    slots = [2, 0, 3, -1, 1]
     T = sum(lens)
     x = rnd((T, channels + 6), 1)
     w = rnd((channels, taps), 2, 0.6)
