@@ -67,7 +67,7 @@ LOTO_R = {
     "architecture": "Lotorax", "vocab": 160, "width": 64, "embedding": {"scale": 8.0}, "norm": {"eps": 1e-5},
     "layers": [
         {"type": "latent_attention", "mixer": _latent(4, 32, 16, 48, 64, base=10000.0, scaling=YARN), "mlp": _moe(32, 8, 2)},
-        {"type": "delta", "mixer": _delta(4, 2, 32, 64, 4), "mlp": _dense(96)},
+        {"type": "delta", "mixer": _delta(4, 2, 16, 80, 3), "mlp": _dense(104)},
     ],
     "loop": {"start": 0, "stop": 2, "times": 1},
 }
