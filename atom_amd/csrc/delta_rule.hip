@@ -220,27 +220,48 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     }
     __syncthreads();
     if (t0 + kRun < end) load_run(t0 + kRun);
+    // a token's k and q entries are read from LDS one token ahead of their use, so that the chain below never
+    // waits for them
+    float kc[kDPL], qc[kDPL], kn[kDPL], qn[kDPL];
+#pragma unroll
+    for (int e = 0; e < kDPL; ++e) {
+      kc[e] = ks[0][e * LPC + sub];
+      qc[e] = qs[0][e * LPC + sub];
+    }
 #pragma unroll
     for (int j = 0; j < kRun; ++j) {
-      if (j >= n) break;
+      if (j < n) {
       const float g = gs[j], beta = bs[j];
       const float v = vv[j];
+      if (j + 1 < kRun) {
+#pragma unroll
+        for (int e = 0; e < kDPL; ++e) {
+          kn[e] = ks[j + 1][e * LPC + sub];
+          qn[e] = qs[j + 1][e * LPC + sub];
+        }
+      }
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int e = 0; e < kDPL; ++e) {
         S[e] *= g;
-        part[e & 3] = fmaf(S[e], ks[j][e * LPC + sub], part[e & 3]);
+        part[e & 3] = fmaf(S[e], kc[e], part[e & 3]);
       }
       const float dot = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
       const float u = beta * (v - dot);
       part[0] = part[1] = part[2] = part[3] = 0.f;
 #pragma unroll
       for (int e = 0; e < kDPL; ++e) {
-        S[e] = fmaf(ks[j][e * LPC + sub], u, S[e]);
-        part[e & 3] = fmaf(S[e], qs[j][e * LPC + sub], part[e & 3]);
+        S[e] = fmaf(kc[e], u, S[e]);
+        part[e & 3] = fmaf(S[e], qc[e], part[e & 3]);
       }
       const float o = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
       if (live && sub == 0) out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
+#pragma unroll
+      for (int e = 0; e < kDPL; ++e) {
+        kc[e] = kn[e];
+        qc[e] = qn[e];
+      }
+      }
     }
   }
 #pragma unroll

@@ -40,25 +40,26 @@ def i32(values):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [48, 200, 1031])
-def test_layernorm_modes(dtype, width):
+@pytest.mark.parametrize("width,n", [(48, 7), (200, 7), (1031, 7), (200, 300), (5000, 7), (1031, 260)])
+def test_layernorm_modes(dtype, width, n):
+    """Few rows and wide rows (a block a row), many rows (a wave a row)."""
     ops = gpu_ops()
-    x = (rnd((7, width), 1, 2.0) + 0.7).to(dtype)
+    x = (rnd((n, width), 1, 2.0) + 0.7).to(dtype)
     w, b, w2, b2 = 1 + rnd((width,), 2, 0.2), rnd((width,), 3, 0.3), 1 + rnd((width,), 4, 0.2), rnd((width,), 5, 0.3)
     dev = lambda t: t.to(DEV)  # noqa: E731
     eps = 3e-5
-    out = torch.empty((7, width), dtype=dtype, device=DEV)
+    out = torch.empty((n, width), dtype=dtype, device=DEV)
     close(ops.layernorm(dev(x), dev(w), dev(b), eps, out), pl.layer_norm(x.double(), w.double(), b.double(), eps), dtype, "plain")
-    res = torch.empty((7, width), dtype=torch.float32, device=DEV)
+    res = torch.empty((n, width), dtype=torch.float32, device=DEV)
     ops.layernorm(dev(x), dev(w), dev(b), eps, out, residual=res, mode="init")
     assert torch.equal(res.cpu(), x.float())
-    y = rnd((7, width), 6).to(dtype)
+    y = rnd((n, width), 6).to(dtype)
     ops.layernorm(dev(y), dev(w), dev(b), eps, out, residual=res, mode="add")
     total = x.double() + y.double()
     close(res, total, torch.float32, "sum")
     close(out, pl.layer_norm(total, w.double(), b.double(), eps), dtype, "add")
     # the normed rows join the stream unrounded, and the stream is normed for what follows
-    z = rnd((7, width), 7, 3.0).to(dtype)
+    z = rnd((n, width), 7, 3.0).to(dtype)
     ops.layernorm(dev(z), dev(w), dev(b), eps, out, residual=res, mode="post", next_weight=dev(w2), next_bias=dev(b2))
     total = total + pl.layer_norm(z.double(), w.double(), b.double(), eps)
     close(res, total, torch.float32, "post sum")
@@ -70,7 +71,7 @@ def test_layernorm_modes(dtype, width):
     assert torch.equal(res, before)
     close(few, pl.layer_norm((total + y.double())[[5, 0, 5]], w.double(), b.double(), eps), dtype, "rows")
     # a float32 input (the stream's own summand) with an output of the serving type
-    f32 = torch.empty((7, width), dtype=torch.float32, device=DEV)
+    f32 = torch.empty((n, width), dtype=torch.float32, device=DEV)
     close(ops.layernorm(dev(x.float()), dev(w), dev(b), eps, f32), pl.layer_norm(x.double(), w.double(), b.double(), eps),
           torch.float32, "float32 out")
 
