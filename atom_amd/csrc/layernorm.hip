@@ -2,9 +2,8 @@
 //
 //   y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * w + b          all in float32
 //
-// The variance is the two-pass one (mean, then the mean of the squared deviations).  From 256 rows on, rows of up to
-// 4,096 entries take a wave each and stay in registers; fewer or wider rows take a block each and sit in LDS
-// between the passes.
+// One block per row; the row sits in LDS as float32 between the passes (mean, then the mean of the
+// squared deviations, then the output), so the variance is the two-pass one.
 //
 // modes of atom_layernorm:
 //   0 plain  y = LN(x)
@@ -74,93 +73,6 @@ layernorm_kernel(const TX* __restrict__ x, float* __restrict__ residual, const f
   for (int i = tid; i < width; i += kNormThreads) yr[i] = from_f32<TY>((row[i] - mean) * rstd * w2[i] + b2[i]);
 }
 
-// The same norm with a wave per row and the row in registers (VPL values a lane): no barrier, the two sums of a
-// norm are two exchanges across the wave.  For widths up to 64 * 64.
-template <typename TX, typename TY, int VPL>
-__global__ void __launch_bounds__(256)
-layernorm_wave_kernel(const TX* __restrict__ x, float* __restrict__ residual, const float* __restrict__ w,
-                      const float* __restrict__ b, const float* __restrict__ w2, const float* __restrict__ b2,
-                      TY* __restrict__ y, const int* __restrict__ rows, int num_rows, int width, float eps, int mode) {
-  const int dst_row = blockIdx.x * 4 + threadIdx.x / kWave;
-  if (dst_row >= num_rows) return;
-  const int lane = threadIdx.x % kWave;
-  const size_t src = rows ? (size_t)rows[dst_row] : (size_t)dst_row;
-  const TX* xr = x + src * width;
-  float* rr = residual ? residual + src * width : nullptr;
-  const float inv_width = 1.f / (float)width;
-  float v[VPL];
-  float part = 0.f;
-#pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    const int i = lane + j * kWave;
-    v[j] = 0.f;
-    if (i < width) {
-      v[j] = to_f32(xr[i]);
-      if (mode == 2) v[j] += rr[i];
-      part += v[j];
-    }
-  }
-  if (mode == 1 || (mode == 2 && rows == nullptr)) {
-#pragma unroll
-    for (int j = 0; j < VPL; ++j)
-      if (lane + j * kWave < width) rr[lane + j * kWave] = v[j];
-  }
-  float mean = wave_sum(part) * inv_width;
-  part = 0.f;
-#pragma unroll
-  for (int j = 0; j < VPL; ++j)
-    if (lane + j * kWave < width) part += (v[j] - mean) * (v[j] - mean);
-  float rstd = 1.f / sqrtf(wave_sum(part) * inv_width + eps);
-  if (mode != 3) {
-    TY* yr = y + (size_t)dst_row * width;
-#pragma unroll
-    for (int j = 0; j < VPL; ++j) {
-      const int i = lane + j * kWave;
-      if (i < width) yr[i] = from_f32<TY>((v[j] - mean) * rstd * w[i] + b[i]);
-    }
-    return;
-  }
-  part = 0.f;
-#pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    const int i = lane + j * kWave;
-    if (i < width) {
-      v[j] = rr[i] + ((v[j] - mean) * rstd * w[i] + b[i]);
-      rr[i] = v[j];
-      part += v[j];
-    }
-  }
-  if (y == nullptr) return;
-  mean = wave_sum(part) * inv_width;
-  part = 0.f;
-#pragma unroll
-  for (int j = 0; j < VPL; ++j)
-    if (lane + j * kWave < width) part += (v[j] - mean) * (v[j] - mean);
-  rstd = 1.f / sqrtf(wave_sum(part) * inv_width + eps);
-  TY* yr = y + (size_t)dst_row * width;
-#pragma unroll
-  for (int j = 0; j < VPL; ++j) {
-    const int i = lane + j * kWave;
-    if (i < width) yr[i] = from_f32<TY>((v[j] - mean) * rstd * w2[i] + b2[i]);
-  }
-}
-
-template <typename TX, typename TY>
-static void launch_layernorm_wave(const void* x, float* residual, const float* w, const float* b, const float* w2,
-                                  const float* b2, void* y, const int* rows, int num_rows, int width, float eps,
-                                  int mode, hipStream_t stream) {
-  dim3 grid((num_rows + 3) / 4), block(256);
-#define WAVE_LAUNCH(V)                                                                                          \
-  hipLaunchKernelGGL((layernorm_wave_kernel<TX, TY, V>), grid, block, 0, stream, (const TX*)x, residual, w, b, w2, \
-                     b2, (TY*)y, rows, num_rows, width, eps, mode)
-  if (width <= 4 * kWave) WAVE_LAUNCH(4);
-  else if (width <= 8 * kWave) WAVE_LAUNCH(8);
-  else if (width <= 16 * kWave) WAVE_LAUNCH(16);
-  else if (width <= 32 * kWave) WAVE_LAUNCH(32);
-  else WAVE_LAUNCH(64);
-#undef WAVE_LAUNCH
-}
-
 ATOM_EXPORT int atom_layernorm(const void* x, int x_dtype, float* residual, const float* w, const float* b,
                                const float* w2, const float* b2, void* y, int y_dtype, const int* rows, int num_rows,
                                int width, float eps, int mode, hipStream_t stream) {
@@ -173,16 +85,6 @@ ATOM_EXPORT int atom_layernorm(const void* x, int x_dtype, float* residual, cons
   if ((unsigned)x_dtype > 1u || (unsigned)y_dtype > 1u) return ATOM_BAD_DTYPE;
   if ((size_t)(width + 16) * sizeof(float) > 160 * 1024) return ATOM_TOO_LARGE;
   if (num_rows == 0) return ATOM_OK;
-  // many rows: a wave each; few rows: a block each, whose 256 threads keep more loads in flight per row
-  if (width <= 64 * kWave && num_rows >= 256) {
-    switch (x_dtype * 2 + y_dtype) {
-      case 0: launch_layernorm_wave<float, float>(x, residual, w, b, w2, b2, y, rows, num_rows, width, eps, mode, stream); break;
-      case 1: launch_layernorm_wave<float, bf16_t>(x, residual, w, b, w2, b2, y, rows, num_rows, width, eps, mode, stream); break;
-      case 2: launch_layernorm_wave<bf16_t, float>(x, residual, w, b, w2, b2, y, rows, num_rows, width, eps, mode, stream); break;
-      default: launch_layernorm_wave<bf16_t, bf16_t>(x, residual, w, b, w2, b2, y, rows, num_rows, width, eps, mode, stream); break;
-    }
-    return launch_status();
-  }
   const size_t smem = (size_t)(width + 16) * sizeof(float);
   dim3 grid(num_rows), block(kNormThreads);
 #define LAUNCH(TX, TY)                                                                                       \
