@@ -206,7 +206,9 @@ __global__ void __launch_bounds__(256) latent_mfma_kernel(LatentParams p) {
     __syncthreads();   // the chunk before has been read
     stash(c);
     __syncthreads();
-    if (c + 1 < my_hi) fetch(c + 1);
+    // not inside a branch: the compiler waits for loads that a branch issued where the branch ends.  Past the last
+    // chunk the last one is read again and never staged.
+    fetch(c + 1 < my_hi ? c + 1 : my_hi - 1);
     if (!wave_busy) continue;
 
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
