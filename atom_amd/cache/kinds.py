@@ -64,6 +64,11 @@ class CacheKind:
         """Paged kinds: how many of the latest tokens a later query can still see (None: all)."""
         return None
 
+    def chunk(self, need) -> int | None:
+        """Paged kinds: a later query sees only what its own run of this many positions (counted from position 0)
+        holds (None: no such limit)."""
+        return None
+
     def keeps_every_token(self, need) -> bool:
         """True if everything a request's earlier tokens left is still there later, in pages: only then
         can a new request take over pages that already hold its beginning (the prefix cache)."""
@@ -95,8 +100,11 @@ class PagedKeysValues(CacheKind):
     def window(self, need):
         return need.window
 
+    def chunk(self, need):
+        return need.chunk
+
     def keeps_every_token(self, need):
-        return need.window is None
+        return need.window is None and need.chunk is None
 
     def page_bytes(self, need, page_size, dtype):
         return 2 * need.num_kv_heads * need.head_dim * page_size * _elem_size(dtype)

@@ -48,6 +48,11 @@ class GroupSpec:
     page_size: int
     num_pages: int
     window: int | None = None  # None: every key is kept
+    chunk: int | None = None   # a query sees only its own run of this many positions, counted from position 0
+
+    @property
+    def keeps_all(self) -> bool:
+        return self.window is None and self.chunk is None
 
 
 class PagePool:
@@ -178,7 +183,7 @@ class CacheManager:
     def __init__(self, groups: list[GroupSpec], num_state_slots: int, prefix_caching: bool = False):
         if not groups:
             groups = []
-        if prefix_caching and any(g.window is not None for g in groups):
+        if prefix_caching and any(not g.keeps_all for g in groups):
             raise ValueError("the prefix cache needs groups that keep every key")
         if prefix_caching and len({g.page_size for g in groups}) > 1:
             raise ValueError("the prefix cache needs one page size")
@@ -188,6 +193,8 @@ class CacheManager:
                 raise ValueError(f"bad group {g}")
             if g.window is not None and g.window <= 0:
                 raise ValueError("a window must be positive")
+            if g.chunk is not None and g.chunk <= 0:
+                raise ValueError("a chunk must be positive")
         self.groups = list(groups)
         self.pools = [PagePool(g.num_pages) for g in groups]
         self.slots = StateSlots(num_state_slots)
@@ -238,14 +245,17 @@ class CacheManager:
     def _first_page_needed(self, group: int, cached: int) -> int:
         """Index of the first page a query at position >= ``cached`` can still see."""
         g = self.groups[group]
-        if g.window is None:
-            return 0
-        return max(0, cached - g.window + 1) // g.page_size
+        first = 0
+        if g.window is not None:
+            first = max(0, cached - g.window + 1)
+        if g.chunk is not None:
+            first = max(first, cached // g.chunk * g.chunk)   # the chunk of the next position begins here
+        return first // g.page_size
 
     def _end_for(self, group: int, upto: int, reserve: int | None) -> int:
         # groups that keep every key may reserve beyond this step (the whole prompt at
         # admission); a window group holds only what the step needs
-        if reserve is not None and self.groups[group].window is None:
+        if reserve is not None and self.groups[group].keeps_all:
             return max(upto, reserve)
         return upto
 
@@ -261,7 +271,7 @@ class CacheManager:
                 continue
             last = (end - 1) // g.page_size
             table = req.tables[gi] if req else []
-            if g.window is None:
+            if g.keeps_all:
                 # nothing is given back before the request ends: the table has no gaps
                 out.append(max(0, last + 1 - len(table)))
                 continue
@@ -289,7 +299,7 @@ class CacheManager:
                 continue
             last = (end - 1) // g.page_size
             table = req.tables[gi]
-            if g.window is None:
+            if g.keeps_all:
                 while len(table) <= last:
                     table.append(self.pools[gi].take())
                 continue
@@ -375,7 +385,7 @@ class CacheManager:
                 raise AssertionError(f"request {req_id!r}: {len(req.tokens)} tokens noted, {cached_after} in the cache")
             self._publish(req, cached_after)
         for gi, g in enumerate(self.groups):
-            if g.window is None:
+            if g.keeps_all:
                 continue
             first = self._first_page_needed(gi, cached_after)
             table = req.tables[gi]

@@ -30,15 +30,21 @@ class CachePlan:
 
 
 def group_runs(model) -> tuple[list[int | None], list[int | None]]:
-    """(window of each group, group of each run).  Runs whose mixers keep pages with the same
-    window share a group, that is, block tables."""
-    windows: list[int | None] = []
+    """(window of each group, group of each run); see ``group_horizons``."""
+    horizons, run_group = group_horizons(model)
+    return [w for w, _ in horizons], run_group
+
+
+def group_horizons(model) -> tuple[list[tuple], list[int | None]]:
+    """((window, chunk) of each group, group of each run).  Runs whose mixers keep pages with the same
+    window and chunk share a group, that is, block tables."""
+    windows: list[tuple] = []
     run_group: list[int | None] = []
     for run in model.order:
         need = model.blocks[run.layer].mixer.cache_need()
         kind = kind_of(need)
         if kind is not None and kind.paged:
-            window = kind.window(need)
+            window = (kind.window(need), kind.chunk(need))
             if window not in windows:
                 windows.append(window)
             run_group.append(windows.index(window))
@@ -51,7 +57,7 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
                budget_bytes: int | None = None, max_num_seqs: int = 1, max_model_len: int = 0,
                max_num_batched_tokens: int = 0) -> CachePlan:
     """Either ``num_pages`` for every group, or a byte budget to divide."""
-    windows, run_group = group_runs(model)
+    windows, run_group = group_horizons(model)
     per_page = [0] * len(windows)
     per_slot = 0
     for run, group in zip(model.order, run_group):
@@ -70,6 +76,9 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
         per_slot += kind.request_bytes(need, dtype)
         if group is not None:
             per_page[group] += kind.page_bytes(need, page_size, dtype)
+    need = model.embedding.cache_need()
+    if need is not None:
+        per_slot += kind_of(need).request_bytes(need, dtype)
     if num_pages is not None:
         counts = [num_pages] * len(windows)
     else:
@@ -78,18 +87,19 @@ def plan_cache(model, page_size: int, dtype: torch.dtype, *, num_pages: int | No
         full_pages = -(-max_model_len // page_size)
         counts = [0] * len(windows)
         left = budget_bytes - per_slot * max_num_seqs
-        for gi, w in enumerate(windows):
-            if w is None:
+        for gi, (w, c) in enumerate(windows):
+            if w is None and c is None:
                 continue
-            per_req = min(full_pages, -(-(w + max_num_batched_tokens) // page_size) + 1)
+            reach = min(x for x in (w, c) if x is not None)   # positions before a step's first that it can see
+            per_req = min(full_pages, -(-(reach + max_num_batched_tokens) // page_size) + 1)
             counts[gi] = per_req * max_num_seqs
             left -= counts[gi] * per_page[gi]
-        full = [gi for gi, w in enumerate(windows) if w is None]
+        full = [gi for gi, (w, c) in enumerate(windows) if w is None and c is None]
         if full:
             pages = max(0, left) // max(1, sum(per_page[gi] for gi in full))
             for gi in full:
                 counts[gi] = pages
-    groups = [GroupSpec(page_size, c, w) for c, w in zip(counts, windows)]
+    groups = [GroupSpec(page_size, n, w, c) for n, (w, c) in zip(counts, windows)]
     return CachePlan(groups, run_group, per_page, per_slot)
 
 
@@ -119,6 +129,16 @@ class CacheStorage:
                                     dtype=dtype)
             self.bindings.append(binding)
             self._owned.append((kind, binding))
+        # an embedding that keeps something per request (its previous token, say) gets a binding of its own
+        self.embedding_binding = None
+        need = model.embedding.cache_need()
+        if need is not None:
+            kind = kind_of(need)
+            if kind.paged:
+                raise ValueError("an embedding's memory is per request, not paged")
+            self.embedding_binding = kind.allocate(need, group=None, num_pages=0, page_size=0,
+                                                   num_slots=num_state_slots, device=device, dtype=dtype)
+            self._owned.append((kind, self.embedding_binding))
         # kinds that clear something when a request starts (the others inherit the base's empty method)
         self._resettable = [(k, b) for k, b in self._owned if type(k).reset is not CacheKind.reset]
 

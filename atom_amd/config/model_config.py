@@ -294,6 +294,127 @@ class LotoraxConfig(ModelConfig):
         return out
 
 
+@dataclass(frozen=True)
+class RalitarConfig(ModelConfig):
+    """``Ralitar``: a token embedding plus a hashed bigram embedding; layers listed one by one, each a mixer (a
+    real-gated linear recurrence, the gated delta rule with a decay per key channel, or chunked attention whose
+    values are its keys) and an optional dense feed-forward, RMS-normed on their way into the stream, then a small
+    per-layer input that depends on the token itself.  config.json keys: ``vocab``, ``width``, ``norm.eps``,
+    ``embedding.bigram`` (``buckets``, ``mul_prev``, ``mul_cur``), ``token_side.dim``, ``layers`` (``type``,
+    ``mixer``, ``mlp``)."""
+
+    layers: tuple = ()
+    norm_eps: float = 1e-6
+    bigram: tuple | None = None       # (buckets, mul_prev, mul_cur)
+    side_dim: int = 0                 # columns of the per-layer token input (0: the model has none)
+
+    model_type: ClassVar[str] = "ralitar"
+    MIXER_TYPES: ClassVar[tuple] = ("rglru", "channel_delta", "attention")
+    MLP_KINDS: ClassVar[tuple] = ("dense",)
+
+    @classmethod
+    def from_dict(cls, raw: dict) -> "RalitarConfig":
+        layers = _need(raw, "layers", list, "the model")
+        bigram = (raw.get("embedding") or {}).get("bigram")
+        if bigram is not None:
+            bigram = tuple(_need(bigram, k, int, "'embedding.bigram'") for k in ("buckets", "mul_prev", "mul_cur"))
+        side = raw.get("token_side")
+        cfg = cls(
+            architecture=raw.get("architecture") or (raw.get("architectures") or ["Ralitar"])[0],
+            vocab_size=_need(raw, "vocab", int, "the model"),
+            hidden_size=_need(raw, "width", int, "the model"),
+            num_hidden_layers=len(layers),
+            max_position_embeddings=_take(raw, "max_position_embeddings", int, 1 << 20),
+            tie_word_embeddings=False,
+            torch_dtype=str(raw.get("torch_dtype") or raw.get("dtype") or "bfloat16"),
+            bos_token_id=raw.get("bos_token_id"),
+            eos_token_id=raw.get("eos_token_id"),
+            layers=tuple(layers),
+            norm_eps=_need(raw.get("norm"), "eps", float, "'norm'"),
+            bigram=bigram,
+            side_dim=_need(side, "dim", int, "'token_side'") if side is not None else 0,
+        )
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size <= 0 or self.hidden_size <= 0 or not self.layers:
+            raise ConfigError("vocab, width and the number of layers must be positive")
+        if self.norm_eps <= 0:
+            raise ConfigError("norm.eps must be positive")
+        if self.bigram is not None and self.bigram[0] <= 0:
+            raise ConfigError("embedding.bigram.buckets must be positive")
+        if self.side_dim < 0:
+            raise ConfigError("token_side.dim must not be negative")
+
+        def positive(m, keys, where):
+            for key in keys:
+                if _need(m, key, int, where) <= 0:
+                    raise ConfigError(f"{where}: {key} must be positive")
+
+        for i, layer in enumerate(self.layers):
+            where = f"layer {i}"
+            kind = _need(layer, "type", str, where)
+            if kind not in self.MIXER_TYPES:
+                raise ConfigError(f"{where}: unknown type {kind!r}; known: {self.MIXER_TYPES}")
+            m = _need(layer, "mixer", dict, where)
+            mw = f"{where}'s mixer"
+            if kind == "rglru":
+                positive(m, ("width", "blocks", "conv"), mw)
+                if m["width"] % m["blocks"]:
+                    raise ConfigError(f"{where}: width must be a multiple of blocks")
+            elif kind == "channel_delta":
+                positive(m, ("heads", "kv_heads", "dim", "vdim", "conv"), mw)
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
+            else:
+                positive(m, ("heads", "kv_heads", "dim", "vdim"), mw)
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"{where}: heads must be a multiple of kv_heads")
+                if m["vdim"] != m["dim"]:
+                    raise ConfigError(f"{where}: the values are the keys, so vdim must equal dim")
+                _need(m, "scale", float, mw)
+                if m.get("softcap") is not None and _need(m, "softcap", float, mw) <= 0:
+                    raise ConfigError(f"{where}: softcap must be positive")
+                mask = m.get("mask")
+                if mask is not None and _need(mask, "size", int, f"{where}'s mask") <= 0:
+                    raise ConfigError(f"{where}: mask.size must be positive")
+                rot = m.get("rot")
+                if rot is not None:
+                    dims = _need(rot, "dims", int, f"{where}'s rot")
+                    _need(rot, "base", float, f"{where}'s rot")
+                    if dims % 2 or dims < 0 or dims > m["dim"]:
+                        raise ConfigError(f"{where}: rot.dims must be even and at most dim")
+                    if rot.get("scaling") is not None:
+                        for key in ("factor", "low", "high", "original"):
+                            _need(rot["scaling"], key, float, f"{where}'s rot.scaling")
+                        if rot["scaling"]["high"] == rot["scaling"]["low"]:
+                            raise ConfigError(f"{where}: rot.scaling needs high and low to differ")
+            mlp = layer.get("mlp")
+            if mlp is not None:
+                mk = _need(mlp, "kind", str, f"{where}'s mlp")
+                if mk not in self.MLP_KINDS:
+                    raise ConfigError(f"{where}: unknown mlp kind {mk!r}; known: {self.MLP_KINDS}")
+                positive(mlp, ("ff",), f"{where}'s mlp")
+
+    def to_dict(self) -> dict:
+        out: dict[str, Any] = {
+            "architecture": self.architecture, "model_type": self.model_type, "vocab": self.vocab_size,
+            "width": self.hidden_size, "norm": {"eps": self.norm_eps},
+            "layers": [dict(layer) for layer in self.layers],
+        }
+        if self.bigram is not None:
+            out["embedding"] = {"bigram": dict(zip(("buckets", "mul_prev", "mul_cur"), self.bigram))}
+        if self.side_dim:
+            out["token_side"] = {"dim": self.side_dim}
+        if self.max_position_embeddings != 1 << 20:
+            out["max_position_embeddings"] = self.max_position_embeddings
+        for key in ("bos_token_id", "eos_token_id"):
+            if getattr(self, key) is not None:
+                out[key] = getattr(self, key)
+        return out
+
+
 def read_config_json(folder: str) -> dict:
     path = os.path.join(folder, "config.json")
     if not os.path.isfile(path):

@@ -7,7 +7,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable
 
-from .model_config import ConfigError, LotoraxConfig, ModelConfig, Qwen3Config
+from .model_config import ConfigError, LotoraxConfig, ModelConfig, Qwen3Config, RalitarConfig
 
 
 @dataclass(frozen=True)
@@ -75,3 +75,7 @@ def _ensure_builtin() -> None:
 
     if "Lotorax" not in _ARCHITECTURES:
         register_architecture("Lotorax", LotoraxConfig, lotorax_spec)
+    from ..models.ralitar import ralitar_spec
+
+    if "Ralitar" not in _ARCHITECTURES:
+        register_architecture("Ralitar", RalitarConfig, ralitar_spec)

@@ -81,6 +81,10 @@ class StepContext:
     prepared: dict = field(default_factory=dict)
     # a scratch dictionary for parts: what one layer derived from the above and the next can use again
     memo: dict = field(default_factory=dict)
+    # the step's token ids (int32 [T], on the device) and the model's shared token tables by checkpoint prefix,
+    # for parts other than the embedding that look a token up; set by the model before its first layer
+    token_ids: torch.Tensor | None = None
+    tables: dict = field(default_factory=dict)
     # host-side copies, for mixers that walk requests themselves; None in a replayed step
     seq_starts: list[int] | None = None   # first row of each request in the token axis
     seq_lens: list[int] | None = None     # rows of each request in this step

@@ -163,7 +163,8 @@ class EngineCore:
             logits = self.graphs.run(entries, cached_now)
         else:
             ctx, token_ids, want_rows = self._build(entries, order)
-            logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows)
+            logits = self.model.forward(ctx, token_ids, self.storage.bindings, want_rows,
+                                        self.storage.embedding_binding)
 
         for e in entries:
             self.lengths[e.req_id] += len(e.tokens)

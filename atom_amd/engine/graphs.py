@@ -211,7 +211,7 @@ class DecodeGraphs:
                 slot_arrays[gi][first:first + k] = mgr.slot_mapping(e.req_id, gi, c, k)
                 bt, state = tables[gi], cap.row_state[gi]
                 held, serial = state[row], mgr.serial(e.req_id)
-                windowed = mgr.groups[gi].window is not None
+                windowed = not mgr.groups[gi].keeps_all
                 if table[(c + k - 1) // page_size] < 0:
                     raise AssertionError(f"request {e.req_id!r}: position {c + k - 1} has no page")
                 if not windowed and held is not None and held[0] == serial and held[1] <= len(table):
@@ -276,7 +276,8 @@ class DecodeGraphs:
         stream.wait_stream(torch.cuda.current_stream(core.device))
         with torch.cuda.stream(stream):
             core.ops.feed_tokens(tokens, feed, core.sampled)
-            core.model.forward(ctx, tokens, core.storage.bindings, want)   # first-use allocations happen here
+            # first-use allocations happen here
+            core.model.forward(ctx, tokens, core.storage.bindings, want, core.storage.embedding_binding)
         stream.synchronize()
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
@@ -292,7 +293,8 @@ class DecodeGraphs:
             with torch.cuda.graph(cap.graph, pool=self.pool, stream=stream):
                 # rows whose token the last step's sampler left on the device take it from there
                 core.ops.feed_tokens(tokens, feed, core.sampled)
-                cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want)
+                cap.logits = core.model.forward(ctx, tokens, core.storage.bindings, want,
+                                                core.storage.embedding_binding)
         finally:
             if gc_was_enabled:
                 gc.enable()

@@ -160,7 +160,7 @@ class LLMEngine:
         """How many requests the pages hold at once, by context length
         (the reference's table, atom/model_engine/model_runner.py:1751-1781)."""
         cfg = self.config
-        full = [g for g in self.core.plan.groups if g.window is None]
+        full = [g for g in self.core.plan.groups if g.keeps_all]
         if not full:
             return
         pages, page = min(g.num_pages for g in full), full[0].page_size

@@ -120,7 +120,7 @@ class Scheduler:
         if not self.enable_chunked_prefill and n > self.max_num_batched_tokens:
             return f"{n} tokens exceed max_num_batched_tokens {self.max_num_batched_tokens} with chunked prefill off"
         for gi, g in enumerate(self.manager.groups):
-            if g.window is None:
+            if g.keeps_all:
                 need = -(-n // g.page_size)
                 if need > g.num_pages:
                     return f"needs {need} cache pages, the pool has {g.num_pages}"

@@ -40,6 +40,9 @@ class ModelSpec:
     # hidden_size); it is handed the stream and the embedding's output
     join: PartChoice | None = None
     join_prefix: str = "join"
+    # further tables with a row per token id that parts of several layers read (kinds from the EMBEDDINGS registry,
+    # built with the checkpoint prefix they are listed under); a part finds them in ``ctx.tables[prefix]``
+    tables: dict[str, PartChoice] = field(default_factory=dict)
     max_positions: int = 0
     embedding_prefix: str = "model.embed_tokens"
     layer_prefix: str = "model.layers.{}"
@@ -68,6 +71,7 @@ class CausalLM(Part):
                                     tied_to=self.embedding if spec.tie_word_embeddings else None,
                                     prefix=spec.head_prefix)
         self.join = spec.join.build(JOINS, hidden_size=spec.hidden_size, prefix=spec.join_prefix) if spec.join else None
+        self.tables = {prefix: choice.build(EMBEDDINGS, prefix=prefix) for prefix, choice in spec.tables.items()}
         self.order = spec.running_order()
         if self.join is None and any(run.enters for run in self.order):
             raise ValueError("a run is marked as the start of a pass, but the model names no join")
@@ -92,8 +96,8 @@ class CausalLM(Part):
         self.device: torch.device | None = None
 
     def children(self):
-        return [self.embedding, *([self.join] if self.join is not None else []), *self.blocks, self.final_norm,
-                self.head]
+        return [self.embedding, *self.tables.values(), *([self.join] if self.join is not None else []), *self.blocks,
+                self.final_norm, self.head]
 
     def drops(self, name: str) -> str | None:
         """Why a checkpoint tensor that no parameter names is left aside without an error, or None if it
@@ -119,10 +123,16 @@ class CausalLM(Part):
     def vocab_size(self) -> int:
         return self.spec.vocab_size
 
-    def forward(self, ctx, token_ids: torch.Tensor, caches: list, want_rows: torch.Tensor | None):
+    def forward(self, ctx, token_ids: torch.Tensor, caches: list, want_rows: torch.Tensor | None,
+                embedding_cache=None):
         """Runs the step's tokens through every run of the order; returns float32 logits
-        at ``want_rows`` (None: nothing is wanted, the cache is only filled)."""
-        hidden = first = self.embedding.forward(ctx, token_ids)
+        at ``want_rows`` (None: nothing is wanted, the cache is only filled).  ``embedding_cache`` is the binding
+        of an embedding that keeps something per request."""
+        ctx.token_ids, ctx.tables = token_ids, self.tables
+        if self.embedding.cache_need() is not None:
+            hidden = first = self.embedding.forward(ctx, token_ids, embedding_cache)
+        else:
+            hidden = first = self.embedding.forward(ctx, token_ids)
         residual = None
         for run, cache in zip(self.order, caches):
             if run.enters:

@@ -92,6 +92,11 @@ class Part:
             return self.prefix
         return f"{self.prefix}.{local}" if self.prefix else local
 
+    def adopt_shapes(self, shape_of) -> None:
+        """Called by the loader before the parameters are declared: ``shape_of(local name)`` is the shape of that
+        checkpoint tensor under this part's prefix, or None if the checkpoint has none.  A part whose sizes are not
+        all in the configuration (an inner size of a product of two matrices, say) takes them from here."""
+
     def finalize(self, device, dtype) -> None:
         """Called once after the parameters are bound; builds derived tables."""
 
@@ -104,11 +109,13 @@ class Part:
 
 @dataclass(frozen=True)
 class KVCacheNeed:
-    """A mixer that keeps keys and values of past tokens in pages.  ``window`` None = all keys."""
+    """A mixer that keeps keys and values of past tokens in pages.  ``window`` None = all keys; ``chunk``: a
+    query sees only the keys of its own run of ``chunk`` positions, counted from position 0."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    chunk: int | None = None
 
 
 @dataclass(frozen=True)
@@ -157,6 +164,11 @@ class PositionEncoding(Part):
 class Embedding(Part):
     """Token ids to the model's first hidden rows.  Built with ``vocab_size``, ``hidden_size`` and whatever
     else its choice names (a multiplier, say)."""
+
+    def cache_need(self):
+        """What the embedding keeps per request between steps (a ``StateNeed``), or None.  An embedding with a
+        need is called as ``forward(ctx, ids, cache)`` with the binding the engine made for it."""
+        return None
 
     def forward(self, ctx, ids: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError

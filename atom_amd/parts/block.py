@@ -94,5 +94,62 @@ class SandwichBlock(Block):
         return self.ffn_post.forward(ctx, out, out_dtype=torch.float32), residual
 
 
+class PostNormBlock(Block):
+    """Norms on the sublayers' outputs only: ``x += norm1(mixer(x))``, then ``x += norm2(ffn(x))``
+    (``feed_forward`` None leaves it out), then, where the layer has one, a ``side`` part (kind from the
+    FEED_FORWARDS registry) that is handed the stream and adds to it itself.  The sublayers read the stream, which
+    is float32; the block keeps it whole (nothing pending) and hands it on as ``hidden`` with no residual.  A
+    copy of the stream in the step's type, for the products that read it, comes out of the kernel that adds to
+    it."""
+
+    def __init__(self, mixer: PartChoice, feed_forward: PartChoice | None, norm: PartChoice,
+                 side: PartChoice | None = None, prefix: str = "", names: dict[str, str] | None = None):
+        super().__init__(prefix)
+        n = {"mixer": "mix", "mixer_post": "norm1", "ffn": "mlp", "ffn_post": "norm2", "side": "side", **(names or {})}
+        sub = lambda name: f"{prefix}.{n[name]}" if prefix else n[name]  # noqa: E731
+        self._mixer = mixer.build(MIXERS, prefix=sub("mixer"))
+        self.mixer_post = norm.build(NORMS, prefix=sub("mixer_post"))
+        self.ffn = feed_forward.build(FEED_FORWARDS, prefix=sub("ffn")) if feed_forward is not None else None
+        self.ffn_post = norm.build(NORMS, prefix=sub("ffn_post")) if self.ffn is not None else None
+        self.side = side.build(FEED_FORWARDS, prefix=sub("side")) if side is not None else None
+        for post in (self.mixer_post, self.ffn_post):
+            if post is not None and not hasattr(post, "forward_post"):
+                raise ValueError(f"{type(post).__name__} cannot add its output to the stream (no forward_post)")
+
+    @property
+    def mixer(self):
+        return self._mixer
+
+    def children(self):
+        parts = [self._mixer, self.mixer_post]
+        if self.ffn is not None:
+            parts += [self.ffn, self.ffn_post]
+        if self.side is not None:
+            parts.append(self.side)
+        return parts
+
+    def forward(self, ctx, hidden, residual, cache):
+        ops = ctx.ops
+        if residual is not None:
+            raise ValueError("this block takes the whole stream, with nothing pending beside it")
+        stream = ops.materialize(hidden)
+        if stream.dtype != torch.float32:
+            raise ValueError("this block keeps a float32 stream: the embedding before it must write float32")
+        # the stream in the step's type, as the products read it: left by the block before this one, or made now
+        reads = ctx.memo.pop(("stream copy", stream.data_ptr()), None)
+        if reads is None:
+            reads = stream if ctx.dtype == torch.float32 else ops.cast_rows(stream, ctx.dtype)
+        mixed = ops.materialize(self._mixer.forward(ctx, reads, cache))
+        reads = self.mixer_post.forward_post(ctx, mixed, stream)
+        if self.ffn is not None:
+            out = ops.materialize(self.ffn.forward(ctx, reads))
+            reads = self.ffn_post.forward_post(ctx, out, stream)
+        if self.side is not None:
+            reads = self.side.forward_stream(ctx, reads, stream)
+        ctx.memo[("stream copy", stream.data_ptr())] = reads
+        return stream, None
+
+
 BLOCKS.register("prenorm", PreNormBlock)
 BLOCKS.register("sandwich", SandwichBlock)
+BLOCKS.register("postnorm", PostNormBlock)

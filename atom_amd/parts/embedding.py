@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamSpec
+from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamSpec, StateNeed
 
 
 class TokenEmbedding(Embedding):
@@ -38,6 +38,37 @@ class ScaledEmbedding(TokenEmbedding):
         return ctx.ops.embedding_scaled(self.params["weight"], ids, out, self.scale)
 
 
+class BigramEmbedding(TokenEmbedding):
+    """``table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets]`` as float32 rows; a request's
+    first token, which has no previous one, takes row ``buckets`` (the last) of ``pairs``.  The previous token of a
+    request's next token is part of its state: an int32 per state slot that holds the last token + 1 (0, what a
+    fresh slot holds: none yet), so that single tokens and portions cut anywhere find it, also in a replayed graph
+    whose token ids exist on the device only."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int, prefix: str = "",
+                 weight_name: str = "weight", bigram_name: str = "bigram"):
+        super().__init__(vocab_size, hidden_size, prefix, weight_name)
+        if buckets <= 0:
+            raise ValueError("the pair table needs at least one bucket")
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.bigram_name = bigram_name
+
+    def param_specs(self):
+        return {**super().param_specs(),
+                "pairs": ParamSpec.single(self.bigram_name, (self.buckets + 1, self.hidden_size))}
+
+    def cache_need(self):
+        return StateNeed((1,), torch.int32)
+
+    def forward(self, ctx, ids: torch.Tensor, cache=None) -> torch.Tensor:
+        if cache is None:
+            raise ValueError("the pair embedding needs its per-request state (the previous token)")
+        out = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
+        return ctx.ops.embedding_bigram(self.params["weight"], self.params["pairs"], ids, cache.state,
+                                        ctx.cu_seqlens_q, ctx.slot_of_seq, ctx.token_seq, out, self.buckets,
+                                        self.mul_prev, self.mul_cur)
+
+
 class LMHead(Head):
     """``logits = x @ W.T`` in float32 out.  ``tied_to`` names the embedding whose table it shares."""
 
@@ -64,4 +95,5 @@ class LMHead(Head):
 
 EMBEDDINGS.register("token_embedding", TokenEmbedding)
 EMBEDDINGS.register("scaled_f32_embedding", ScaledEmbedding)
+EMBEDDINGS.register("bigram_embedding", BigramEmbedding)
 HEADS.register("lm_head", LMHead)

@@ -13,13 +13,23 @@ from .base import NORMS, Norm, ParamSpec
 class RMSNorm(Norm):
     accepts_deferred = True   # the kernel adds the slices of a product that is still a sum
 
-    def __init__(self, size: int, eps: float, prefix: str = ""):
+    def __init__(self, size: int, eps: float, prefix: str = "", weight_name: str = "weight"):
         super().__init__(prefix)
         self.size = size
         self.eps = float(eps)
+        self.weight_name = weight_name   # the checkpoint's name under the prefix (empty: the prefix itself)
 
     def param_specs(self):
-        return {"weight": ParamSpec.single("weight", (self.size,), kind="vector", init="one_plus_normal")}
+        return {"weight": ParamSpec.single(self.weight_name, (self.size,), kind="vector", init="one_plus_normal")}
+
+    def forward_post(self, ctx, x, stream, copy: bool = True):
+        """``stream += norm(x)`` in float32, nothing rounded on the way; returns the stream's rows in the step's
+        type for the sublayer that reads them next (``copy`` False, or a float32 step: the stream itself)."""
+        out = None
+        if copy and ctx.dtype != torch.float32:
+            out = torch.empty(tuple(stream.shape), dtype=ctx.dtype, device=stream.device)
+        ctx.ops.rmsnorm_post(x, self.params["weight"], self.eps, stream, out)
+        return stream if out is None else out
 
     def forward(self, ctx, x):
         out = torch.empty(tuple(x.shape), dtype=x.dtype, device=x.device)
@@ -47,6 +57,10 @@ class RMSNorm(Norm):
             lazy = pending(x, residual, self.params["weight"], self.eps, rows)
             if lazy is not None:
                 return lazy
+        if residual is None and x.dtype == torch.float32 and ctx.dtype != torch.float32:
+            # a float32 stream with nothing pending, normed into the step's type
+            out = torch.empty((rows.numel(), self.size), dtype=ctx.dtype, device=x.device)
+            return ctx.ops.rmsnorm_rows(x, self.params["weight"], self.eps, rows, out)
         out = torch.empty((rows.numel(), self.size), dtype=x.dtype, device=x.device)
         mode = "add" if residual is not None else "plain"
         return ctx.ops.rmsnorm(x, self.params["weight"], self.eps, out, residual=residual, mode=mode, rows=rows)

@@ -88,5 +88,49 @@ class ScaledRotary(PositionEncoding):
         self.freq = freq.to(device)
 
 
+class BandedRotary(PositionEncoding):
+    """Rotation of interleaved pairs (2i, 2i + 1) of the first ``dims`` entries by ``position * f_i``,
+    ``f_i = base^(-2i / dims)``, with the frequencies scaled by the band their wavelength ``l = 2 pi / f`` falls in
+    (the scheme of the Llama 3.1 models): unchanged where ``l < original / high``, divided by ``factor`` where
+    ``l > original / low``, and between the two ``(1 - s) f / factor + s f`` with ``s = (original / l - low) /
+    (high - low)``.  Without ``factor`` the frequencies are plain.
+
+    Offers what ``ScaledRotary`` offers: ``freq`` (float64 [dims / 2], on the device), ``mult`` (1 here) and
+    ``dims``; kernels form the angle in float64 from the position, so there is no table and no position limit."""
+
+    def __init__(self, dims: int, base: float, factor: float | None = None, low: float | None = None,
+                 high: float | None = None, original: float | None = None, head_dim: int | None = None,
+                 prefix: str = ""):
+        super().__init__(prefix)
+        if dims % 2 or dims < 0 or (head_dim is not None and dims > head_dim):
+            raise ValueError(f"rotated dimensions come in pairs within a head, got {dims}")
+        self.dims = int(dims)
+        self.base = float(base)
+        self.scaling = None
+        if factor is not None:
+            if None in (low, high, original):
+                raise ValueError("banded scaling needs factor, low, high and original")
+            if float(high) == float(low):
+                raise ValueError("banded scaling needs high and low to differ")
+            self.scaling = (float(factor), float(low), float(high), float(original))
+        self.freq: torch.Tensor | None = None
+        self.mult = 1.0
+
+    def frequencies(self) -> torch.Tensor:
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        f = self.base ** (-2.0 * i / max(self.dims, 1))
+        if self.scaling is None:
+            return f
+        factor, low, high, original = self.scaling
+        length = 2 * math.pi / f
+        s = (original / length - low) / (high - low)
+        between = (1 - s) * f / factor + s * f
+        return torch.where(length < original / high, f, torch.where(length > original / low, f / factor, between))
+
+    def finalize(self, device, dtype):
+        self.freq = self.frequencies().to(device)
+
+
 POSITION_ENCODINGS.register("rotary", RotaryEncoding)
 POSITION_ENCODINGS.register("scaled_rotary", ScaledRotary)
+POSITION_ENCODINGS.register("banded_rotary", BandedRotary)

@@ -154,8 +154,11 @@ def expected_tensors(model: Part) -> dict[str, tuple[tuple[int, ...], ParamSpec]
 def load_weights(model: Part, source: TensorSource, device, dtype: torch.dtype,
                  progress: Callable[[str], None] | None = None) -> None:
     """Fills every declared parameter of ``model`` from ``source`` or raises ``WeightError``."""
-    expected = expected_tensors(model)
     present = set(source.names())
+    for part in model.walk():
+        part.adopt_shapes(lambda local, part=part: tuple(source.shape(part.full_name(local)))
+                          if part.full_name(local) in present else None)
+    expected = expected_tensors(model)
     drops = getattr(model, "drops", None)
     missing = [n for n in expected if n not in present]
     unexpected = []
@@ -178,7 +181,9 @@ def load_weights(model: Part, source: TensorSource, device, dtype: torch.dtype,
             stored = {source.dtype(part.full_name(s.name)) for s in spec.sources}
             widest = torch.float32 if (torch.float32 in stored or torch.float64 in stored) else next(iter(stored))
             target = param_dtype(spec, widest, dtype)
-            param = torch.empty(spec.shape, dtype=target, device=device)
+            # zeros: a parameter's sources need not cover all its rows (a bias that only some of the stacked
+            # products have)
+            param = torch.zeros(spec.shape, dtype=target, device=device)
             for s in spec.sources:
                 tensor = source.get(part.full_name(s.name))
                 param[s.offset:s.offset + s.rows].copy_(tensor.to(device=device, dtype=target), non_blocking=False)

@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 
 import plain_lotorax as pl
+import plain_ralitar as pr
 from plain_model import causal_attention, exponential_race, rms_norm, rope_neox, silu_and_mul, top_k_top_p_filter
 
 WIDE = torch.float64
@@ -78,9 +79,11 @@ class PlainKernels:
     def attention_tile_rows(self, dtype, head_dim, page_size, group, max_q_len):
         return 0, 0   # this attention walks tokens, it wants no tiles listed
 
-    def paged_attention(self, q, k_cache, v_cache, out, meta, scale, window=None, parts=None):
+    def paged_attention(self, q, k_cache, v_cache, out, meta, scale, window=None, parts=None, softcap=None,
+                        chunk=None):
         tokens, hq, d = q.shape
         page_size = k_cache.shape[2]
+        hkv = k_cache.shape[1]
         for t in range(tokens):
             seq = int(meta.token_seq[t])
             if seq < 0:
@@ -88,11 +91,19 @@ class PlainKernels:
                 continue
             pos = int(meta.positions[t])
             first = max(0, pos - window + 1) if window else 0
+            if chunk:
+                first = max(first, pos // chunk * chunk)
             keys = torch.arange(first, pos + 1)
             pages = meta.block_tables[seq].long()[keys // page_size]
             offs = keys % page_size
             k = k_cache[pages, :, offs, :].to(WIDE)        # [n, hkv, d]
             v = v_cache[pages, :, :, offs].to(WIDE)        # [n, hkv, d]
+            if softcap:
+                for h in range(hq):
+                    s = (k[:, h // (hq // hkv)] @ q[t, h].to(WIDE)) * scale
+                    s = softcap * torch.tanh(s / softcap)
+                    out[t, h] = (torch.softmax(s, dim=0) @ v[:, h // (hq // hkv)]).to(out.dtype)
+                continue
             o = causal_attention(q[t:t + 1].to(WIDE), k, v, scale, None, torch.tensor([pos]), keys)
             out[t] = o[0].to(out.dtype)
         return out
@@ -179,7 +190,7 @@ class PlainKernels:
         return q_abs
 
     def heads_gemm(self, x, x_offset, ldx, hsx, weight, y, y_offset, ldy, hsy, heads, m, n, k, alpha=1.0, gate=None,
-                   gate_offset=0, ldg=0):
+                   gate_offset=0, ldg=0, exact=False):
         xf, yf = x.reshape(-1), y.view(-1)
         for h in range(heads):
             xs = torch.as_strided(xf, (m, k), (ldx, 1), x_offset + h * hsx).to(WIDE)
@@ -213,7 +224,8 @@ class PlainKernels:
             out[t] = ((e / denom) @ rows[:, :rank]).to(out.dtype)
         return out
 
-    def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out, max_q_len=None):
+    def conv_silu_state(self, x, channels, taps_weight, state, cu_seqlens_q, slot_of_seq, out, max_q_len=None,
+                        bias=None, activation="silu"):
         taps = taps_weight.shape[1]
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
@@ -222,12 +234,21 @@ class PlainKernels:
                 continue
             tail = state[slot, :(taps - 1) * channels].view(taps - 1, channels)
             y, new_tail = pl.short_convolution(x[lo:hi, :channels].to(WIDE), taps_weight.to(WIDE), tail.to(WIDE))
-            out[lo:hi] = pl.silu(y).to(out.dtype)
+            if bias is not None:
+                y = y + bias.to(WIDE)
+            out[lo:hi] = (pl.silu(y) if activation == "silu" else y).to(out.dtype)
             tail.copy_(new_tail.to(tail.dtype))
         return out
 
     def delta_rule(self, qkv, gates, a_off, b_off, a_log, dt_bias, state, state_off, cu_seqlens_q, slot_of_seq, out,
-                   heads, kv_heads, dim, vdim):
+                   heads, kv_heads, dim, vdim, decay=None, per_channel=False):
+        if per_channel:
+            return self._delta_rule_channels(qkv, gates, a_off, b_off, a_log, dt_bias, state, state_off, cu_seqlens_q,
+                                             slot_of_seq, out, heads, kv_heads, dim, vdim,
+                                             gates if decay is None else decay)
+        if decay is not None:
+            gates = torch.cat((gates, decay), dim=1)
+            a_off = gates.shape[1] - decay.shape[1] + a_off
         for b in range(slot_of_seq.numel()):
             lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
             if slot < 0:
@@ -251,11 +272,124 @@ class PlainKernels:
                 S[h] = new.to(S.dtype)
         return out
 
-    def delta_out(self, o, gates, gate_off, weight, eps, out):
+    def _delta_rule_channels(self, qkv, gates, a_off, b_off, a_log, dt_bias, state, state_off, cu_seqlens_q,
+                             slot_of_seq, out, heads, kv_heads, dim, vdim, decay):
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            n = hi - lo
+            x = qkv[lo:hi].to(WIDE)
+            q = x[:, :kv_heads * dim].reshape(n, kv_heads, dim)
+            k = x[:, kv_heads * dim:2 * kv_heads * dim].reshape(n, kv_heads, dim)
+            v = x[:, 2 * kv_heads * dim:].reshape(n, heads, vdim)
+            q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dim ** -0.5
+            k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+            beta = torch.sigmoid(gates[lo:hi, b_off:b_off + heads].to(WIDE))
+            raw = decay[lo:hi, a_off:a_off + heads * dim].to(WIDE) + dt_bias.to(WIDE)
+            g = torch.exp(-torch.exp(a_log.to(WIDE)).view(1, heads, 1) * pr.softplus(raw).view(n, heads, dim))
+            S = state[slot, state_off:state_off + heads * dim * vdim].view(heads, dim, vdim)
+            for h in range(heads):
+                kv = h // (heads // kv_heads)
+                cur = S[h].to(WIDE)
+                for t in range(n):
+                    o, cur = pr.delta_step(cur, q[t, kv], k[t, kv], v[t, h], beta[t, h], g[t, h])
+                    out[lo + t, h] = o.to(out.dtype)
+                S[h] = cur.to(S.dtype)
+        return out
+
+    def delta_out(self, o, gates, gate_off, weight, eps, out, activation="silu"):
         tokens, heads, vdim = o.shape
         g = gates[:, gate_off:gate_off + heads * vdim].to(WIDE).view(tokens, heads, vdim)
-        y = pl.rms_unit(o.to(WIDE), eps) * weight.to(WIDE) * pl.silu(g)
+        y = pl.rms_unit(o.to(WIDE), eps) * weight.to(WIDE) * (pl.silu(g) if activation == "silu" else torch.sigmoid(g))
         out.copy_(y.reshape(tokens, heads * vdim).to(out.dtype))
+        return out
+
+    # ---- the kernels of the float32-stream block, the pair embedding, the gated recurrence and key-value attention
+
+    def embedding_bigram(self, table, pairs, ids, state, cu_seqlens_q, slot_of_seq, token_seq, out, buckets, mul_prev,
+                         mul_cur):
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if hi <= lo:
+                continue
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            prev = int(state[slot, 0]) - 1
+            for t in range(lo, hi):
+                cur = int(ids[t])
+                row = buckets if prev < 0 else (prev * mul_prev + cur * mul_cur) % buckets
+                out[t] = (table[cur].to(WIDE) + pairs[row].to(WIDE)).to(out.dtype)
+                prev = cur
+            state[slot, 0] = prev + 1
+        return out
+
+    def rmsnorm_post(self, x, weight, eps, stream, out=None):
+        stream.copy_((stream.to(WIDE) + pr.rms(x.to(WIDE), eps) * weight.to(WIDE)).to(stream.dtype))
+        if out is not None:
+            out.copy_(stream.to(out.dtype))
+        return out
+
+    def rmsnorm_rows(self, x, weight, eps, rows, out):
+        out.copy_((pr.rms(x[rows.long()].to(WIDE), eps) * weight.to(WIDE)).to(out.dtype))
+        return out
+
+    def cast_rows(self, x, dtype):
+        return x.to(dtype)
+
+    def token_gate(self, raw, table, col_off, ids, out):
+        e = table[ids.long(), col_off:col_off + raw.shape[1]].to(WIDE)
+        out.copy_((pr.gelu_tanh(raw.to(WIDE)) * e).to(out.dtype))
+        return out
+
+    def rglru_scan(self, u, gates, ra_bias, ri_bias, lam, proj, y_off, state, state_off, cu_seqlens_q, slot_of_seq, out,
+                   decay_scale):
+        c = u.shape[1]
+        sp = pr.softplus(lam.to(WIDE))
+        for b in range(slot_of_seq.numel()):
+            lo, hi, slot = int(cu_seqlens_q[b]), int(cu_seqlens_q[b + 1]), int(slot_of_seq[b])
+            if slot < 0:
+                out[lo:hi] = 0
+                continue
+            S = state[slot, state_off:state_off + c].to(WIDE)
+            for t in range(lo, hi):
+                r = torch.sigmoid(gates[0, t].to(WIDE) + ra_bias.to(WIDE).reshape(-1))
+                i = torch.sigmoid(gates[1, t].to(WIDE) + ri_bias.to(WIDE).reshape(-1))
+                a = torch.exp(-decay_scale * r * sp)
+                S = a * S + torch.sqrt(1 - a * a) * (i * u[t].to(WIDE))
+                out[t] = (S * pr.gelu_tanh(proj[t, y_off:y_off + c].to(WIDE))).to(out.dtype)
+            state[slot, state_off:state_off + c] = S.to(state.dtype)
+        return out
+
+    def keys_as_values_write(self, proj, q_out, k_cache, v_cache, q_weight, k_weight, freq, rot_dims, positions, slots,
+                             num_heads, num_kv_heads, head_dim, page_size, eps, write_kv=True):
+        t = proj.shape[0]
+        qn, kn = num_heads * head_dim, num_kv_heads * head_dim
+        q, k = proj[:, :qn].to(WIDE), proj[:, qn:qn + kn].to(WIDE)
+        v = k.reshape(t, num_kv_heads, head_dim)
+        if q_weight is not None:
+            q = pr.rms(q, eps) * q_weight.to(WIDE)
+        if k_weight is not None:
+            k = pr.rms(k, eps) * k_weight.to(WIDE)
+        q, k = q.reshape(t, num_heads, head_dim), k.reshape(t, num_kv_heads, head_dim)
+        if rot_dims:
+            q, k = pr.rotate_pairs(q, positions, freq.to(WIDE)), pr.rotate_pairs(k, positions, freq.to(WIDE))
+        q_out.copy_(q.to(q_out.dtype))
+        if write_kv:
+            for i in range(t):
+                slot = int(slots[i])
+                if slot < 0:
+                    continue
+                page, off = divmod(slot, page_size)
+                k_cache[page, :, off, :] = k[i].to(k_cache.dtype)
+                v_cache[page, :, :, off] = v[i].to(v_cache.dtype)
+        return q_out
+
+    def sigmoid_gate(self, x, gates, gate_off, out):
+        g = gates[:, gate_off:gate_off + x.shape[1]].to(WIDE)
+        out.copy_((x.to(WIDE) * torch.sigmoid(g)).to(out.dtype))
         return out
 
     def router_choose(self, logits, correction, top, renormalize=False):
