@@ -3,7 +3,8 @@
 //
 // One block per (query token, query head).  The token's request and absolute position
 // are given per token; the keys it sees are positions max(0, p - window + 1) .. p of that
-// request, found through the request's block table.  Keys are walked in fixed chunks
+// request, found through the request's block table; with `chunk` only those from the start of the run of `chunk`
+// positions (counted from position 0) that p lies in.  With `softcap` a score s becomes softcap * tanh(s / softcap).  Keys are walked in fixed chunks
 // counted from position 0 with a running maximum and sum (all float32), so the result
 // for a token depends only on its own keys: not on the batch, not on how the prompt
 // was cut into steps, not on which pages hold the keys.
@@ -20,7 +21,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_
                                const T* __restrict__ v_cache, T* __restrict__ out,
                                const int* __restrict__ token_seq, const int* __restrict__ positions,
                                const int* __restrict__ block_tables, int max_blocks, int hq, int hkv,
-                               int d, int page_size, float scale, int window) {
+                               int d, int page_size, float scale, int window, int chunk, float softcap) {
   extern __shared__ float smem[];
   float* qs = smem;                  // d
   float* probs = qs + d;             // kAttnChunk
@@ -41,7 +42,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_
   for (int i = tid; i < d; i += kAttnThreads) qs[i] = to_f32(qr[i]) * scale;
   __syncthreads();
 
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (chunk > 0 && pos / chunk * chunk > first) first = pos / chunk * chunk;
   const int last = pos;  // inclusive
   // each thread owns output dims tid, tid + 128, ... (at most 4 for d <= 512)
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -61,6 +63,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k_
       const T* kr = k_cache + (((size_t)page * hkv + kvh) * page_size + off) * (size_t)d;
       float s = 0.f;
       for (int i = 0; i < d; ++i) s += qs[i] * to_f32(kr[i]);
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       probs[j] = s;
       local_max = fmaxf(local_max, s);
     }
@@ -104,9 +107,9 @@ ATOM_EXPORT int atom_paged_attention_generic(const void* q, const void* k_cache,
                                              const int* token_seq, const int* positions,
                                              const int* block_tables, int max_blocks, int dtype, int tokens,
                                              int hq, int hkv, int d, int page_size, float scale, int window,
-                                             hipStream_t stream) {
+                                             int chunk, float softcap, hipStream_t stream) {
   if (tokens < 0 || hq <= 0 || hkv <= 0 || d <= 0 || page_size <= 0 || max_blocks <= 0) return ATOM_BAD_SHAPE;
-  if (hq % hkv) return ATOM_BAD_SHAPE;
+  if (hq % hkv || window < 0 || chunk < 0 || softcap < 0.f) return ATOM_BAD_SHAPE;
   if (d > 4 * kAttnThreads) return ATOM_TOO_LARGE;
   if (hq > 65535) return ATOM_TOO_LARGE;
   if (tokens == 0) return ATOM_OK;
@@ -115,6 +118,6 @@ ATOM_EXPORT int atom_paged_attention_generic(const void* q, const void* k_cache,
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((paged_attention_generic_kernel<T>), grid, block, smem, stream,
                                                  (const T*)q, (const T*)k_cache, (const T*)v_cache, (T*)out,
                                                  token_seq, positions, block_tables, max_blocks, hq, hkv, d,
-                                                 page_size, scale, window));
+                                                 page_size, scale, window, chunk, softcap));
   return launch_status();
 }

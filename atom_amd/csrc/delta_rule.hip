@@ -10,14 +10,15 @@
 // Requests are walked through the step's device arrays (cu_seqlens_q, slot_of_seq), so the same kernels serve
 // prompt portions, single tokens and padded rows (slot < 0: nothing is read or written) of a replayed graph.
 //
-//   conv_silu_state   one thread per (request, channel, run of 64 tokens)
+//   conv_silu_state   one thread per (request, channel, run of 64 tokens); optionally a bias per channel, and SiLU or
+//                     no activation
 //   delta_rule        blocks per (request, head, group of columns); a column of S (over dim) sits in the registers of up
 //                     to 16 adjacent lanes, so the columns never meet; q, k and the gates of a run of tokens are
 //                     staged in LDS
-//   delta_out         o / rms(o) * w * silu(gate), rounded to the serving type
+//   delta_out         o / rms(o) * w * silu(gate) (or sigmoid(gate)), rounded to the serving type
 #include "common.h"
 
-constexpr int kMaxTaps = 8;
+constexpr int kMaxTaps = 16;
 
 constexpr int kConvRun = 64;   // tokens of a request that one block takes
 
@@ -27,7 +28,8 @@ template <typename TW>
 __global__ void __launch_bounds__(256)
 conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restrict__ taps_w, int taps, int channels,
                        float* __restrict__ state, long slot_stride, const int* __restrict__ cu_seqlens,
-                       const int* __restrict__ slot_of_seq, float* __restrict__ y) {
+                       const int* __restrict__ slot_of_seq, float* __restrict__ y, const float* __restrict__ bias,
+                       int act) {
   const int c = blockIdx.x * 256 + threadIdx.x;
   const int seq = blockIdx.y;
   if (c >= channels) return;
@@ -46,6 +48,7 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
     w[j] = j < taps ? to_f32(taps_w[(size_t)c * taps + j]) : 0.f;
     win[j] = 0.f;
   }
+  const float b = bias != nullptr ? bias[c] : 0.f;
   float* tail = state + (size_t)slot * slot_stride;   // [taps - 1, channels], oldest first
   // the taps - 1 inputs before `first`: the step's own tokens where there are enough, else the carried ones
 #pragma unroll
@@ -66,7 +69,8 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
 #pragma unroll
     for (int j = 0; j < kMaxTaps; ++j)
       if (j < taps) s = fmaf(w[j], win[j], s);
-    y[(size_t)t * channels + c] = s / (1.f + expf(-s));
+    s += b;
+    y[(size_t)t * channels + c] = act == 0 ? s / (1.f + expf(-s)) : s;
   }
   if (blockIdx.z == 0) {
     // the request's last taps - 1 inputs after this step
@@ -89,8 +93,10 @@ conv_silu_state_kernel(const float* __restrict__ x, int ldx, const TW* __restric
 
 ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w, int w_dtype, int taps, int channels,
                                      float* state, long slot_stride, const int* cu_seqlens, const int* slot_of_seq,
-                                     int num_seqs, int max_q_len, float* y, hipStream_t stream) {
+                                     int num_seqs, int max_q_len, float* y, const float* bias, int act,
+                                     hipStream_t stream) {
   if (taps < 1 || taps > kMaxTaps) return ATOM_TOO_LARGE;
+  if (act != 0 && act != 1) return ATOM_UNSUPPORTED;   // 0: SiLU, 1: none
   if (channels <= 0 || ldx < channels || num_seqs < 0 || slot_stride < (long)(taps - 1) * channels) return ATOM_BAD_SHAPE;
   if (x == nullptr || taps_w == nullptr || state == nullptr || y == nullptr || max_q_len < 0) return ATOM_BAD_SHAPE;
   if (num_seqs == 0) return ATOM_OK;
@@ -99,7 +105,7 @@ ATOM_EXPORT int atom_conv_silu_state(const float* x, int ldx, const void* taps_w
   dim3 grid((channels + 255) / 256, num_seqs, runs), block(256);
   ATOM_DISPATCH_DTYPE(w_dtype, hipLaunchKernelGGL((conv_silu_state_kernel<T>), grid, block, 0, stream, x, ldx,
                                                    (const T*)taps_w, taps, channels, state, slot_stride, cu_seqlens,
-                                                   slot_of_seq, y));
+                                                   slot_of_seq, y, bias, act));
   return launch_status();
 }
 
@@ -129,9 +135,13 @@ constexpr int kDPL = 16;   // entries of a column of S that one lane holds
 // ab [T, ld_ab] float32: the raw decay inputs at a_off and the raw beta inputs at b_off, one per head.
 // A column of S (dim entries) is spread over LPC adjacent lanes, entry i in lane i % LPC, so that a token costs each
 // lane 16 entries and two sums over the LPC lanes; the sums over a lane's entries run in four independent chains.
-template <int LPC>
+//
+// CHANNEL: the decay is one number per head and key channel (row of S): dec holds heads x dim raw inputs a token at
+// a_off, dt_bias heads x dim entries, and a run's decays are staged like its q and k rows.
+template <int LPC, bool CHANNEL>
 __global__ void __launch_bounds__(256)
-delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab, int a_off,
+delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab,
+                  const float* __restrict__ dec, int ld_dec, int a_off,
                   int b_off, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
                   float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
                   const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads, int kv_heads, int dim,
@@ -139,6 +149,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   constexpr int DMAX = kDPL * LPC;
   __shared__ float qs[kRun][DMAX];
   __shared__ float ks[kRun][DMAX];
+  __shared__ float gv[CHANNEL ? kRun : 1][DMAX];   // CHANNEL: a run's decays per key channel
   __shared__ float gs[kRun], bs[kRun];
   const int head = blockIdx.x, seq = blockIdx.y;
   const int tid = threadIdx.x;
@@ -161,7 +172,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     S[j] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
   }
   const float decay_rate = -expf(a_log[head]);
-  const float bias = dt_bias[head];
+  const float bias = CHANNEL ? 0.f : dt_bias[head];
   const float q_scale = 1.f / sqrtf((float)dim);
   const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -169,7 +180,8 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   // are filled for the next run while this run's tokens are worked through, so that no load is waited for inside
   // the chain of tokens.
   constexpr int QK_ITEMS = 2 * kRun * DMAX / 256;
-  float qk_raw[QK_ITEMS], v_next[kRun], a_next = 0.f, b_next = 0.f;
+  constexpr int G_ITEMS = CHANNEL ? kRun * DMAX / 256 : 1;
+  float qk_raw[QK_ITEMS], g_raw[G_ITEMS], v_next[kRun], a_next = 0.f, b_next = 0.f;
   auto load_run = [&](int t0) {
     const int n = end - t0 < kRun ? end - t0 : kRun;
 #pragma unroll
@@ -182,9 +194,17 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
 #pragma unroll
     for (int j = 0; j < kRun; ++j)
       v_next[j] = (live && j < n) ? qkv[(size_t)(t0 + j) * channels + v_off + head * vdim + col] : 0.f;
+    if constexpr (CHANNEL) {
+#pragma unroll
+      for (int it = 0; it < G_ITEMS; ++it) {
+        const int idx = tid + it * 256;
+        const int j = idx / DMAX, i = idx % DMAX;
+        g_raw[it] = (j < n && i < dim) ? dec[(size_t)(t0 + j) * ld_dec + a_off + head * dim + i] : 0.f;
+      }
+    }
     if (tid < n) {
       const float* r = ab + (size_t)(t0 + tid) * ld_ab;
-      a_next = r[a_off + head];
+      if constexpr (!CHANNEL) a_next = dec[(size_t)(t0 + tid) * ld_dec + a_off + head];
       b_next = r[b_off + head];
     }
   };
@@ -198,10 +218,22 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       const int item = idx / DMAX, i = idx % DMAX;
       ((item & 1) ? ks[item >> 1] : qs[item >> 1])[i] = qk_raw[it];
     }
+    if constexpr (CHANNEL) {
+#pragma unroll
+      for (int it = 0; it < G_ITEMS; ++it) {
+        const int idx = tid + it * 256;
+        const int j = idx / DMAX, i = idx % DMAX;
+        const float z = g_raw[it] + (i < dim ? dt_bias[head * dim + i] : 0.f);
+        const float sp_z = z > 20.f ? z : log1pf(expf(z));
+        gv[j][i] = expf(decay_rate * sp_z);
+      }
+    }
     if (tid < n) {
-      const float z = a_next + bias;
-      const float sp_z = z > 20.f ? z : log1pf(expf(z));
-      gs[tid] = expf(decay_rate * sp_z);
+      if constexpr (!CHANNEL) {
+        const float z = a_next + bias;
+        const float sp_z = z > 20.f ? z : log1pf(expf(z));
+        gs[tid] = expf(decay_rate * sp_z);
+      }
       bs[tid] = 1.f / (1.f + expf(-b_next));
     }
     float vv[kRun];
@@ -231,8 +263,14 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
 #pragma unroll
     for (int j = 0; j < kRun; ++j) {
       if (j < n) {
-      const float g = gs[j], beta = bs[j];
+      const float g = CHANNEL ? 1.f : gs[j];
+      const float beta = bs[j];
       const float v = vv[j];
+      float gc[kDPL];
+      if constexpr (CHANNEL) {
+#pragma unroll
+        for (int e = 0; e < kDPL; ++e) gc[e] = gv[j][e * LPC + sub];
+      }
       if (j + 1 < kRun) {
 #pragma unroll
         for (int e = 0; e < kDPL; ++e) {
@@ -243,7 +281,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int e = 0; e < kDPL; ++e) {
-        S[e] *= g;
+        if constexpr (CHANNEL) S[e] *= gc[e]; else S[e] *= g;
         part[e & 3] = fmaf(S[e], kc[e], part[e & 3]);
       }
       const float dot = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
@@ -271,13 +309,16 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   }
 }
 
-ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab, int ld_ab, int a_off, int b_off,
+ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab, int ld_ab, const float* dec, int ld_dec,
+                                int a_off, int b_off, int per_channel,
                                 const float* a_log, const float* dt_bias, float* state, long slot_stride,
                                 long state_off, const int* cu_seqlens, const int* slot_of_seq, int num_seqs, float* out,
                                 int heads, int kv_heads, int dim, int vdim, hipStream_t stream) {
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || num_seqs < 0) return ATOM_BAD_SHAPE;
   if (channels != 2 * kv_heads * dim + heads * vdim) return ATOM_BAD_SHAPE;
-  if (a_off < 0 || b_off < 0 || a_off + heads > ld_ab || b_off + heads > ld_ab) return ATOM_BAD_SHAPE;
+  if (a_off < 0 || b_off < 0 || b_off + heads > ld_ab) return ATOM_BAD_SHAPE;
+  if (a_off + heads * (per_channel ? dim : 1) > ld_dec) return ATOM_BAD_SHAPE;
+  if (ab == nullptr || dec == nullptr) return ATOM_BAD_SHAPE;
   if (state_off < 0 || slot_stride < state_off + (long)heads * dim * vdim) return ATOM_BAD_SHAPE;
   if (dim > 256) return ATOM_TOO_LARGE;
   if (num_seqs == 0) return ATOM_OK;
@@ -287,9 +328,18 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
   const int cols = 256 / lpc;
   dim3 grid(heads, num_seqs, (vdim + cols - 1) / cols), block(256);
   if (grid.z > 65535) return ATOM_TOO_LARGE;
-#define LAUNCH(L)                                                                                                 \
-  hipLaunchKernelGGL((delta_rule_kernel<L>), grid, block, 0, stream, qkv, channels, ab, ld_ab, a_off, b_off, a_log, \
-                     dt_bias, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim, vdim)
+#define LAUNCH_AS(L, C)                                                                                          \
+  hipLaunchKernelGGL((delta_rule_kernel<L, C>), grid, block, 0, stream, qkv, channels, ab, ld_ab, dec, ld_dec, a_off, \
+                     b_off, a_log, dt_bias, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads,     \
+                     kv_heads, dim, vdim)
+#define LAUNCH(L)                  \
+  do {                             \
+    if (per_channel) {             \
+      LAUNCH_AS(L, true);          \
+    } else {                       \
+      LAUNCH_AS(L, false);         \
+    }                              \
+  } while (0)
   switch (lpc) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
@@ -298,6 +348,7 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
     default: LAUNCH(16); break;
   }
 #undef LAUNCH
+#undef LAUNCH_AS
   return launch_status();
 }
 
@@ -308,7 +359,8 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
 template <typename T>
 __global__ void __launch_bounds__(256)
 delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ld_gate, int gate_off,
-                 const float* __restrict__ w, float eps, T* __restrict__ y, int heads, int vdim, size_t items) {
+                 const float* __restrict__ w, float eps, T* __restrict__ y, int heads, int vdim, size_t items,
+                 int act) {
   const size_t item = (size_t)blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
   if (item >= items) return;
   const int lane = threadIdx.x % kWave;
@@ -322,12 +374,14 @@ delta_out_kernel(const float* __restrict__ o, const float* __restrict__ gate, in
   T* dst = y + item * vdim;
   for (int i = lane; i < vdim; i += kWave) {
     const float g = gr[i];
-    dst[i] = from_f32<T>(src[i] * rstd * w[i] * (g / (1.f + expf(-g))));
+    const float sig = 1.f / (1.f + expf(-g));
+    dst[i] = from_f32<T>(src[i] * rstd * w[i] * (act == 0 ? g * sig : sig));
   }
 }
 
 ATOM_EXPORT int atom_delta_out(const float* o, const float* gate, int ld_gate, int gate_off, const float* w, float eps,
-                               void* y, int dtype, int tokens, int heads, int vdim, hipStream_t stream) {
+                               void* y, int dtype, int tokens, int heads, int vdim, int act, hipStream_t stream) {
+  if (act != 0 && act != 1) return ATOM_UNSUPPORTED;   // 0: SiLU of the gate, 1: its sigmoid
   if (tokens < 0 || heads <= 0 || vdim <= 0 || gate_off < 0 || gate_off + heads * vdim > ld_gate) return ATOM_BAD_SHAPE;
   if (o == nullptr || gate == nullptr || w == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
   const size_t items = (size_t)tokens * heads;
@@ -335,6 +389,6 @@ ATOM_EXPORT int atom_delta_out(const float* o, const float* gate, int ld_gate, i
   const size_t blocks = (items + 3) / 4;
   if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
   ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((delta_out_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, o,
-                                                 gate, ld_gate, gate_off, w, eps, (T*)y, heads, vdim, items));
+                                                 gate, ld_gate, gate_off, w, eps, (T*)y, heads, vdim, items, act));
   return launch_status();
 }

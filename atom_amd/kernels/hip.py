@@ -193,7 +193,9 @@ class HipKernels:
                    "atom_delta_out", "atom_router_choose", "atom_experts_gate_up", "atom_experts_down",
                    "atom_latent_attention_mfma", "atom_latent_mfma_supports", "atom_latent_mfma_tokens_per_tile",
                    "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports",
-                   "atom_heads_gemm_mfma", "atom_heads_gemm_mfma_supports"):
+                   "atom_heads_gemm_mfma", "atom_heads_gemm_mfma_supports", "atom_rmsnorm_post", "atom_rmsnorm_rows",
+                   "atom_cast_rows", "atom_token_gate", "atom_embedding_bigram", "atom_rglru_scan",
+                   "atom_keys_as_values_write", "atom_sigmoid_gate"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -680,7 +682,11 @@ class HipKernels:
         return out
 
     def paged_attention(self, q, k_cache, v_cache, out, meta: AttentionMeta, scale: float,
-                        window: int | None = None, parts: int | None = None):
+                        window: int | None = None, parts: int | None = None, softcap: float | None = None,
+                        chunk: int | None = None):
+        """Attention of the step's queries over the pages.  ``window``: only the latest that many keys;
+        ``chunk``: only the keys of the query's own run of that many positions, counted from position 0;
+        ``softcap``: a score s becomes ``softcap * tanh(s / softcap)``."""
         tokens, hq, d = q.shape
         _, hkv, page_size, _ = k_cache.shape
         dt = q.dtype
@@ -698,13 +704,13 @@ class HipKernels:
         if meta.max_context_len > meta.block_tables.shape[1] * page_size:
             raise KernelError("attention: a context is longer than its block table can name")
         group = hq // hkv
-        if (dt == torch.bfloat16 and self.use_mfma_attention
+        if (dt == torch.bfloat16 and self.use_mfma_attention and not softcap and not chunk
                 and self.lib.atom_attention_mfma_supports(d, page_size, group)):
             return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts)
         self._done("paged_attention", self.lib.atom_paged_attention_generic(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions),
             _ptr(meta.block_tables), meta.block_tables.shape[1], self._code(q), tokens, hq, hkv, d, page_size,
-            ctypes.c_float(scale), int(window or 0), self._stream()))
+            ctypes.c_float(scale), int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0), self._stream()))
         return out
 
     def _library_slices(self, m: int, n: int, k: int) -> int:
@@ -969,10 +975,12 @@ class HipKernels:
         return q_abs
 
     def heads_gemm(self, x, x_offset: int, ldx: int, hsx: int, weight, y, y_offset: int, ldy: int, hsy: int, heads: int,
-                   m: int, n: int, k: int, alpha: float = 1.0, gate=None, gate_offset: int = 0, ldg: int = 0):
+                   m: int, n: int, k: int, alpha: float = 1.0, gate=None, gate_offset: int = 0, ldg: int = 0,
+                   exact: bool = False):
         """One small product per head: ``y[t, h, :n] = alpha * x[t, h, :k] @ weight[h].T`` (times
         ``sigmoid(gate[t, h])`` when given), with ``x`` and ``y`` addressed as flat arrays: element (t, h, i) of x
-        sits at ``x_offset + t * ldx + h * hsx + i``.  ``weight`` is [heads, n, k]."""
+        sits at ``x_offset + t * ldx + h * hsx + i``.  ``weight`` is [heads, n, k].  ``exact``: a float32 input is
+        multiplied as it is (float32 multiply-adds), not rounded for the matrix cores."""
         self._check("per-head input", x, (torch.float32, torch.bfloat16))
         self._check("per-head weight", weight, (torch.float32, torch.bfloat16), (heads, n, k))
         self._check("per-head out", y, (torch.float32, torch.bfloat16))
@@ -989,7 +997,8 @@ class HipKernels:
             gp = ctypes.c_void_p(gate.data_ptr() + 4 * gate_offset)
         xp = ctypes.c_void_p(x.data_ptr() + x.element_size() * x_offset)
         yp = ctypes.c_void_p(y.data_ptr() + y.element_size() * y_offset)
-        if (weight.dtype == torch.bfloat16 and m >= self.heads_mfma_from and self.lib.atom_heads_gemm_mfma_supports(
+        if (weight.dtype == torch.bfloat16 and m >= self.heads_mfma_from and not (exact and x.dtype == torch.float32)
+                and self.lib.atom_heads_gemm_mfma_supports(
                 self._code(x), BF16, ctypes.c_long(x_offset), ctypes.c_long(ldx), ctypes.c_long(hsx), k)):
             # many rows: the same product on the matrix cores (a float32 input is rounded to bfloat16 on the way in)
             self._done("heads_gemm_mfma", self.lib.atom_heads_gemm_mfma(
@@ -1057,8 +1066,9 @@ class HipKernels:
     # ------------------------------------------------------------------ the gated delta rule
 
     def conv_silu_state(self, x, channels: int, taps_weight, state, cu_seqlens_q, slot_of_seq, out,
-                        max_q_len: int | None = None):
-        """Short causal convolution per channel over each request's tokens, then SiLU.  ``x`` float32 [tokens, >=
+                        max_q_len: int | None = None, bias=None, activation: str = "silu"):
+        """Short causal convolution per channel over each request's tokens (plus ``bias`` per channel when given),
+        then SiLU (``activation`` "none": nothing).  ``x`` float32 [tokens, >=
         channels] (the first ``channels`` columns are convolved); ``taps_weight`` [channels, taps], last column the
         current token's; ``state`` float32 [slots, >= (taps - 1) * channels]: a request's last taps - 1 inputs, read
         and written back.  Requests with slot -1 are padding.  ``max_q_len``: the most tokens a request brings (an
@@ -1072,37 +1082,55 @@ class HipKernels:
         self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
         self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
         self._check("convolution out", out, torch.float32, (tokens, channels))
+        if bias is not None:
+            self._check("convolution bias", bias, torch.float32, (channels,))
+        if activation not in ("silu", "none"):
+            raise KernelError(f"conv_silu_state: unknown activation {activation!r}")
+        if ldx < channels or state.shape[1] < (taps - 1) * channels:
+            raise KernelError("conv_silu_state: the input or the state is narrower than the channels need")
         self._done("conv_silu_state", self.lib.atom_conv_silu_state(
             _ptr(x), ldx, _ptr(taps_weight), self._code(taps_weight), taps, channels, _ptr(state),
             ctypes.c_long(state.shape[1]), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
-            tokens if max_q_len is None else min(tokens, max_q_len), _ptr(out), self._stream()))
+            tokens if max_q_len is None else min(tokens, max_q_len), _ptr(out), _ptr(bias),
+            0 if activation == "silu" else 1, self._stream()))
         return out
 
     def delta_rule(self, qkv, gates, a_off: int, b_off: int, a_log, dt_bias, state, state_off: int, cu_seqlens_q,
-                   slot_of_seq, out, heads: int, kv_heads: int, dim: int, vdim: int):
+                   slot_of_seq, out, heads: int, kv_heads: int, dim: int, vdim: int, decay=None,
+                   per_channel: bool = False):
         """The gated delta recurrence over each request's tokens.  ``qkv`` float32 [tokens, 2 kv_heads dim + heads
-        vdim] (q | k | v after convolution and SiLU); ``gates`` float32 [tokens, *] with the raw decay inputs at
-        ``a_off`` and the raw beta inputs at ``b_off``; the heads' matrices [heads, dim, vdim] start at
-        ``state_off`` of a slot's row of ``state``.  ``out`` float32 [tokens, heads, vdim]."""
+        vdim] (q | k | v after convolution and SiLU); ``gates`` float32 [tokens, *] with the raw beta inputs at
+        ``b_off`` and, unless ``decay`` (float32 [tokens, *]) holds them, the raw decay inputs at ``a_off``: one
+        per head, or with ``per_channel`` one per head and key channel (``dt_bias`` likewise); the heads' matrices
+        [heads, dim, vdim] start at ``state_off`` of a slot's row of ``state``.  ``out`` float32 [tokens, heads,
+        vdim]."""
         tokens, channels = qkv.shape
         seqs = slot_of_seq.numel()
+        decay = gates if decay is None else decay
+        wide = heads * (dim if per_channel else 1)
+        self._check("delta decay inputs", decay, torch.float32, (tokens, None))
+        if a_off < 0 or a_off + wide > decay.shape[1]:
+            raise KernelError("delta_rule: the decay inputs do not fit their tensor")
         self._check("delta q|k|v", qkv, torch.float32, (tokens, 2 * kv_heads * dim + heads * vdim))
         self._check("delta gates", gates, torch.float32, (tokens, None))
         self._check("A_log", a_log, torch.float32, (heads,))
-        self._check("dt_bias", dt_bias, torch.float32, (heads,))
+        self._check("dt_bias", dt_bias, torch.float32, (wide,))
         self._check("state", state, torch.float32, (None, None))
         self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
         self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
         self._check("delta out", out, torch.float32, (tokens, heads, vdim))
         self._done("delta_rule", self.lib.atom_delta_rule(
-            _ptr(qkv), channels, _ptr(gates), gates.shape[1], a_off, b_off, _ptr(a_log), _ptr(dt_bias), _ptr(state),
+            _ptr(qkv), channels, _ptr(gates), gates.shape[1], _ptr(decay), decay.shape[1], a_off, b_off,
+            int(bool(per_channel)), _ptr(a_log), _ptr(dt_bias), _ptr(state),
             ctypes.c_long(state.shape[1]), ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
             _ptr(out), heads, kv_heads, dim, vdim, self._stream()))
         return out
 
-    def delta_out(self, o, gates, gate_off: int, weight, eps: float, out):
-        """``out[t, h] = o[t, h] / rms(o[t, h]) * weight * silu(gate[t, h])`` with the gate's rows at ``gate_off``
-        of ``gates`` (float32)."""
+    def delta_out(self, o, gates, gate_off: int, weight, eps: float, out, activation: str = "silu"):
+        """``out[t, h] = o[t, h] / rms(o[t, h]) * weight * silu(gate[t, h])`` (``activation`` "sigmoid": times the
+        gate's sigmoid) with the gate's rows at ``gate_off`` of ``gates`` (float32)."""
+        if activation not in ("silu", "sigmoid"):
+            raise KernelError(f"delta_out: unknown activation {activation!r}")
         tokens, heads, vdim = o.shape
         self._check("read-out", o, torch.float32)
         self._check("gates", gates, torch.float32, (tokens, None))
@@ -1110,7 +1138,153 @@ class HipKernels:
         self._check("gated read-out", out, (torch.float32, torch.bfloat16), (tokens, heads * vdim))
         self._done("delta_out", self.lib.atom_delta_out(
             _ptr(o), _ptr(gates), gates.shape[1], gate_off, _ptr(weight), ctypes.c_float(eps), _ptr(out),
-            self._code(out), tokens, heads, vdim, self._stream()))
+            self._code(out), tokens, heads, vdim, 0 if activation == "silu" else 1, self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ a float32 stream with normed summands
+
+    def rmsnorm_post(self, x, weight, eps: float, stream, out=None):
+        """``stream += x / rms(x) * weight`` in float32 (``stream`` float32, in place); ``out``, when given,
+        receives the stream's new rows in its own type."""
+        x = self.materialize(x)
+        rows, width = x.shape
+        self._check("norm input", x, (torch.float32, torch.bfloat16), (rows, width))
+        self._check("norm weight", weight, torch.float32, (width,))
+        self._check("stream", stream, torch.float32, (rows, width))
+        if out is not None:
+            self._check("stream copy", out, (torch.float32, torch.bfloat16), (rows, width))
+        self._done("rmsnorm_post", self.lib.atom_rmsnorm_post(
+            _ptr(x), self._code(x), _ptr(weight), ctypes.c_float(eps), _ptr(stream), _ptr(out),
+            self._code(out) if out is not None else 0, rows, width, self._stream()))
+        return out
+
+    def rmsnorm_rows(self, x, weight, eps: float, rows, out):
+        """``out[r] = norm(x[rows[r]]) * weight`` for float32 ``x``, written in ``out``'s type."""
+        n, width = x.shape
+        self._check("norm input", x, torch.float32, (n, width))
+        self._check("norm weight", weight, torch.float32, (width,))
+        self._check("norm rows", rows, torch.int32, (None,))
+        self._check("norm out", out, (torch.float32, torch.bfloat16), (rows.numel(), width))
+        self._done("rmsnorm_rows", self.lib.atom_rmsnorm_rows(
+            _ptr(x), _ptr(weight), ctypes.c_float(eps), _ptr(rows), n, _ptr(out), self._code(out), rows.numel(), width,
+            self._stream()))
+        return out
+
+    def cast_rows(self, x, dtype):
+        """Float32 rows in another type."""
+        self._check("rows", x, torch.float32)
+        out = torch.empty(tuple(x.shape), dtype=dtype, device=x.device)
+        self._done("cast_rows", self.lib.atom_cast_rows(_ptr(x), _ptr(out), self._code(out), ctypes.c_long(x.numel()),
+                                                        self._stream()))
+        return out
+
+    def token_gate(self, raw, table, col_off: int, ids, out):
+        """``out[t, j] = gelu_tanh(raw[t, j]) * table[ids[t], col_off + j]``."""
+        tokens, dim = raw.shape
+        self._check("gate input", raw, torch.float32, (tokens, dim))
+        self._check("token table", table, (torch.float32, torch.bfloat16), (None, None))
+        self._check("token ids", ids, torch.int32, (tokens,))
+        self._check("gated rows", out, (torch.float32, torch.bfloat16), (tokens, dim))
+        if col_off < 0 or col_off + dim > table.shape[1]:
+            raise KernelError("token_gate: the columns asked for are not in the table")
+        self._done("token_gate", self.lib.atom_token_gate(
+            _ptr(raw), _ptr(table), self._code(table), table.shape[1], col_off, _ptr(ids), table.shape[0], _ptr(out),
+            self._code(out), tokens, dim, self._stream()))
+        return out
+
+    def embedding_bigram(self, table, pairs, ids, state, cu_seqlens_q, slot_of_seq, token_seq, out, buckets: int,
+                         mul_prev: int, mul_cur: int):
+        """``out[t] = table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets]`` in float32, row
+        ``buckets`` of ``pairs`` for a request's first token.  ``state`` int32 [slots, 1] holds a request's last
+        token + 1 between steps (0: none yet) and is moved on."""
+        vocab, hidden = table.shape
+        tokens, seqs = ids.numel(), slot_of_seq.numel()
+        self._check("embedding table", table, (torch.float32, torch.bfloat16))
+        self._check("pair table", pairs, table.dtype, (buckets + 1, hidden))
+        self._check("token ids", ids, torch.int32, (tokens,))
+        self._check("previous tokens", state, torch.int32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("token_seq", token_seq, torch.int32, (tokens,))
+        self._check("embedding out", out, torch.float32, (tokens, hidden))
+        self._done("embedding_bigram", self.lib.atom_embedding_bigram(
+            _ptr(table), _ptr(pairs), self._code(table), _ptr(ids), _ptr(state), ctypes.c_long(state.shape[1]),
+            _ptr(cu_seqlens_q), _ptr(slot_of_seq), _ptr(token_seq), _ptr(out), tokens, hidden, vocab, buckets,
+            ctypes.c_long(mul_prev), ctypes.c_long(mul_cur), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ the real-gated linear recurrence
+
+    def rglru_scan(self, u, gates, ra_bias, ri_bias, lam, proj, y_off: int, state, state_off: int, cu_seqlens_q,
+                   slot_of_seq, out, decay_scale: float):
+        """``S <- a S + sqrt(1 - a^2) (i u)``, ``out = S * gelu_tanh(y)`` over each request's tokens, with
+        ``r = sigmoid(gates[0] + ra_bias)``, ``i = sigmoid(gates[1] + ri_bias)``, ``a = exp(-decay_scale r
+        softplus(lam))``.  ``u`` float32 [tokens, channels]; ``gates`` float32 [2, tokens, channels]; ``y`` the
+        ``channels`` columns of ``proj`` (float32) from ``y_off``; S at ``state_off`` of a slot's row of ``state``."""
+        tokens, channels = u.shape
+        seqs = slot_of_seq.numel()
+        self._check("recurrence input", u, torch.float32, (tokens, channels))
+        self._check("recurrence gates", gates, torch.float32, (2, tokens, channels))
+        self._check("recurrence gate bias", ra_bias, torch.float32)
+        self._check("input gate bias", ri_bias, torch.float32)
+        if ra_bias.numel() != channels or ri_bias.numel() != channels:
+            raise KernelError("rglru_scan: the gates' biases need one entry per channel")
+        self._check("decay parameter", lam, torch.float32, (channels,))
+        self._check("branches", proj, torch.float32, (tokens, None))
+        self._check("state", state, torch.float32, (None, None))
+        self._check("cu_seqlens_q", cu_seqlens_q, torch.int32, (seqs + 1,))
+        self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
+        self._check("recurrence out", out, (torch.float32, torch.bfloat16), (tokens, channels))
+        gi = ctypes.c_void_p(gates.data_ptr() + 4 * tokens * channels)
+        self._done("rglru_scan", self.lib.atom_rglru_scan(
+            _ptr(u), _ptr(gates), gi, _ptr(ra_bias), _ptr(ri_bias), _ptr(lam), _ptr(proj), proj.shape[1], y_off,
+            _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq),
+            seqs, _ptr(out), self._code(out), channels, ctypes.c_float(decay_scale), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention whose values are its keys
+
+    def keys_as_values_write(self, proj, q_out, k_cache, v_cache, q_weight, k_weight, freq, rot_dims: int, positions,
+                             slots, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, eps: float,
+                             write_kv: bool = True):
+        """From the float32 product ``proj`` [tokens, >= (heads + kv_heads) dim] (q | k | ...): q and k RMS-normed
+        over their whole rows (weights [heads dim] and [kv_heads dim]; None: no norm), pairs (2i, 2i + 1) of the
+        first ``rot_dims`` entries of each head turned by ``position * freq[i]``; q to ``q_out``, the normed and
+        rotated k to the key pages, k as projected to the value pages."""
+        tokens, ld = proj.shape
+        self._check("projections", proj, torch.float32)
+        if ld < (num_heads + num_kv_heads) * head_dim:
+            raise KernelError("keys_as_values_write: the product is narrower than q and k")
+        self._check("q out", q_out, (torch.float32, torch.bfloat16), (tokens, num_heads, head_dim))
+        dt = q_out.dtype
+        if q_weight is not None:
+            self._check("q norm weight", q_weight, torch.float32, (num_heads * head_dim,))
+        if k_weight is not None:
+            self._check("k norm weight", k_weight, torch.float32, (num_kv_heads * head_dim,))
+        if rot_dims:
+            self._check("rotation frequencies", freq, torch.float64, (rot_dims // 2,))
+            self._check("positions", positions, torch.int32, (tokens,))
+        if write_kv:
+            self._check("key pages", k_cache, dt, (None, num_kv_heads, page_size, head_dim))
+            self._check("value pages", v_cache, dt, (k_cache.shape[0], num_kv_heads, head_dim, page_size))
+            self._check("slot mapping", slots, torch.int32, (tokens,))
+        self._done("keys_as_values_write", self.lib.atom_keys_as_values_write(
+            _ptr(proj), ld, _ptr(q_out), _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
+            self._code(q_out), _ptr(q_weight), _ptr(k_weight), _ptr(freq) if rot_dims else None, rot_dims,
+            _ptr(positions) if rot_dims else None, _ptr(slots) if write_kv else None, tokens, num_heads, num_kv_heads,
+            head_dim, page_size, ctypes.c_float(eps), self._stream()))
+        return q_out
+
+    def sigmoid_gate(self, x, gates, gate_off: int, out):
+        """``out = x * sigmoid(gates[:, gate_off : gate_off + width])`` (``gates`` float32)."""
+        rows, width = x.shape
+        self._check("gated input", x, (torch.float32, torch.bfloat16), (rows, width))
+        self._check("gates", gates, torch.float32, (rows, None))
+        self._check("gated out", out, x.dtype, (rows, width))
+        if gate_off < 0 or gate_off + width > gates.shape[1]:
+            raise KernelError("sigmoid_gate: the gate's columns are not in their tensor")
+        self._done("sigmoid_gate", self.lib.atom_sigmoid_gate(
+            _ptr(x), self._code(x), _ptr(gates), gates.shape[1], gate_off, _ptr(out), rows, width, self._stream()))
         return out
 
     # ------------------------------------------------------------------ routed experts
