@@ -42,6 +42,9 @@ struct AttnParams {
   float* ws_o;            // decode: [seqs, Hq, parts, D]
   float* ws_ml;           // decode: [seqs, Hq, parts, 2]
   int max_blocks, hq, hkv, page_size, window, seq_offset, parts, num_tiles;
+  int chunk;              // > 0: a query sees only the keys of its own run of `chunk` positions, counted from 0
+  float cap_in, cap_out;  // cap_out > 0: a raw score s becomes cap_out * tanh(s * cap_in), still in raw units
+                          // (cap_in = scale / cap, cap_out = cap / scale, so that the scale applies afterwards)
   int page_shift;         // log2(page_size) where that is a power of two, else -1
   float scale_log2;       // softmax scale * log2(e)
   // decode with the step before attention folded in: q is not read; the float32 QKV product is
@@ -56,6 +59,17 @@ struct AttnParams {
 };
 
 __device__ __forceinline__ s16x4 as_s16x4(bf16x4 v) { return __builtin_bit_cast(s16x4, v); }
+
+// The first key a query at position `pos` sees: the window's and the chunk's starts, whichever is later.
+__device__ __forceinline__ int first_visible(const AttnParams& p, int pos) {
+  int lo = p.window > 0 ? pos - p.window + 1 : 0;
+  if (p.chunk > 0) lo = max(lo, pos / p.chunk * p.chunk);
+  return max(lo, 0);
+}
+
+__device__ __forceinline__ float capped(const AttnParams& p, float s) {
+  return p.cap_out > 0.f ? p.cap_out * tanhf(s * p.cap_in) : s;
+}
 
 // The keys of one part of a decode row: the row's visible keys are cut into steps of ``step`` keys (what a wave
 // takes per trip) and the steps are dealt out evenly, the first (steps % parts) parts taking one more.  No part is
@@ -130,14 +144,12 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
   // ---- key range of this work item
   int kb, ke;
   if (DECODE) {
-    int vis = 0;
-    if (p.window > 0 && ctx - p.window > 0) vis = (ctx - p.window) & ~15;
+    const int vis = first_visible(p, ctx - 1) & ~15;
     const PartKeys mine = part_keys(ctx - vis, p.parts, part, 16);
     kb = vis + mine.begin;
     ke = min(ctx, vis + mine.end);
   } else {
-    kb = 0;
-    if (p.window > 0 && pos0 - p.window + 1 > 0) kb = (pos0 - p.window + 1) & ~15;
+    kb = first_visible(p, pos0) & ~15;
     ke = pos0 + nrows;   // one past the last row's own position
   }
 
@@ -274,7 +286,7 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
     //      row sees whole (all but the last of a decode row's) is not masked.
     const int first_pos = pos0;                                 // the smallest position among the rows
     const int last_pos = DECODE ? pos0 : pos0 + nrows - 1;
-    const bool whole = k0 + 15 <= min(first_pos, ke - 1) && (p.window <= 0 || k0 >= last_pos - p.window + 1);
+    const bool whole = k0 + 15 <= min(first_pos, ke - 1) && k0 >= first_visible(p, last_pos);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float sc[4];
@@ -282,17 +294,17 @@ __global__ void __launch_bounds__(kWave) attention_mfma_kernel(AttnParams p) {
       if (whole) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          sc[i] = s[rt][i];
+          sc[i] = capped(p, s[rt][i]);
           mx = fmaxf(mx, sc[i]);
         }
       } else {
-        const int hi = min(row_pos[rt], ke - 1);                        // last visible key
-        const int lo = p.window > 0 ? row_pos[rt] - p.window + 1 : 0;   // first visible key
+        const int hi = min(row_pos[rt], ke - 1);          // last visible key
+        const int lo = first_visible(p, row_pos[rt]);     // first visible key
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + 4 * g + i;
           const bool vis = key <= hi && key >= lo && key >= kb;
-          sc[i] = vis ? s[rt][i] : -INFINITY;
+          sc[i] = vis ? capped(p, s[rt][i]) : -INFINITY;
           mx = fmaxf(mx, sc[i]);
         }
       }
@@ -393,8 +405,8 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
   const int* table = p.block_tables + (size_t)seq * p.max_blocks;
   const int ps = p.page_size;
 
-  int vis0 = 0;
-  if (p.window > 0 && ctx - p.window > 0) vis0 = (ctx - p.window) & ~31;
+  const int lo0 = first_visible(p, pos0);
+  const int vis0 = lo0 & ~31;
   const PartKeys mine = part_keys(ctx - vis0, p.parts, part, 32);
   const int kb = vis0 + mine.begin;
   const int ke = min(ctx, vis0 + mine.end);
@@ -586,7 +598,7 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
     __builtin_amdgcn_wave_barrier();
 
     // ---- softmax update; lane holds keys k0 + 8 g + 4 b + i of row r16
-    const bool whole = k0 + 31 <= ke - 1 && (p.window <= 0 || k0 >= pos0 - p.window + 1);
+    const bool whole = k0 + 31 <= ke - 1 && k0 >= lo0;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float sc[8];
@@ -594,16 +606,16 @@ __global__ void __launch_bounds__(TOGETHER ? 8 * kWave : kWave, (D <= 128 ? 2 : 
       if (whole) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          sc[e] = s[rt][e / 4][e % 4];
+          sc[e] = capped(p, s[rt][e / 4][e % 4]);
           mx = fmaxf(mx, sc[e]);
         }
       } else {
-        const int lo = p.window > 0 ? pos0 - p.window + 1 : 0;
+        const int lo = lo0;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int key = k0 + 8 * g + e;
           const bool vis = key < ke && key >= lo;
-          sc[e] = vis ? s[rt][e / 4][e % 4] : -INFINITY;
+          sc[e] = vis ? capped(p, s[rt][e / 4][e % 4]) : -INFINITY;
           mx = fmaxf(mx, sc[e]);
         }
       }
@@ -898,8 +910,7 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
   const int pos0 = pos_block0 + ROWS * sub;         // of this wave's first token
   const int ke = pos_block0 + block_rows;           // one past the last key any row of the block sees
   const int my_ke = pos0 + nrows;
-  int kb = 0;
-  if (p.window > 0 && pos_block0 - p.window + 1 > 0) kb = (pos_block0 - p.window + 1) & ~(TK - 1);
+  const int kb = first_visible(p, pos_block0) & ~(TK - 1);
   const int* table = p.block_tables + (size_t)seq * p.max_blocks;
 
   // ---- this wave's queries
@@ -1045,7 +1056,7 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
     bf16x8 pb[RT][KB / 2];
     float alpha[RT];
     bool rescale = false;
-    const bool whole = k0 + TK - 1 <= min(pos0, ke - 1) && (p.window <= 0 || k0 >= pos0 + nrows - p.window);
+    const bool whole = k0 + TK - 1 <= min(pos0, ke - 1) && k0 >= first_visible(p, pos0 + max(nrows, 1) - 1);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       float sc[4 * KB];
@@ -1055,20 +1066,20 @@ __global__ void __launch_bounds__(256 * KS, (D <= 128 && KS == 1 ? 2 : 1)) atten
         for (int b = 0; b < KB; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            sc[4 * b + i] = s[rt][b][i];
+            sc[4 * b + i] = capped(p, s[rt][b][i]);
             mx = fmaxf(mx, sc[4 * b + i]);
           }
       } else {
         // the visible keys, counted from this lane's first key of the tile: 16 b + i is compared with constants
         const int first = k0 + 4 * g;
         const int hi = min(row_pos[rt], ke - 1) - first;
-        const int lo = (p.window > 0 ? row_pos[rt] - p.window + 1 : 0) - first;
+        const int lo = first_visible(p, row_pos[rt]) - first;
 #pragma unroll
         for (int b = 0; b < KB; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const bool vis = 16 * b + i <= hi && 16 * b + i >= lo;
-            sc[4 * b + i] = vis ? s[rt][b][i] : -INFINITY;
+            sc[4 * b + i] = vis ? capped(p, s[rt][b][i]) : -INFINITY;
             mx = fmaxf(mx, sc[4 * b + i]);
           }
       }
@@ -1255,9 +1266,11 @@ static int check_common(int hq, int hkv, int d, int page_size, int max_blocks) {
 ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const void* v_cache, void* out,
                                       const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
                                       int seq_offset, int seqs, int hq, int hkv, int d, int page_size, float scale,
-                                      int window, int parts, float* ws_o, float* ws_ml, hipStream_t stream) {
+                                      int window, int chunk, float softcap, int parts, float* ws_o, float* ws_ml,
+                                      hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
-  if (seqs < 0 || parts < 1 || seq_offset < 0) return ATOM_BAD_SHAPE;
+  if (seqs < 0 || parts < 1 || seq_offset < 0 || window < 0 || chunk < 0 || softcap < 0.f) return ATOM_BAD_SHAPE;
+  if (softcap > 0.f && !(scale > 0.f)) return ATOM_UNSUPPORTED;
   if (parts > kWave) return ATOM_TOO_LARGE;   // the merge keeps one part per lane
   if (parts > 1 && (!ws_o || !ws_ml)) return ATOM_BAD_SHAPE;
   if (seqs > 65535 || hkv > 65535) return ATOM_TOO_LARGE;
@@ -1267,6 +1280,8 @@ ATOM_EXPORT int atom_attention_decode(const void* q, const void* k_cache, const 
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = nullptr;
   p.ws_o = ws_o; p.ws_ml = ws_ml; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = seq_offset; p.parts = parts; p.scale_log2 = scale * 1.4426950408889634f;
+  p.chunk = chunk;
+  if (softcap > 0.f) { p.cap_in = scale / softcap; p.cap_out = softcap / scale; }
   p.page_shift = page_shift_of(page_size);
 #define CALL(DD) return launch_decode<DD, false>(p, seqs, stream)
   ATOM_FOR_HEAD_DIM(d, CALL)
@@ -1323,15 +1338,19 @@ ATOM_EXPORT int atom_attention_decode_fused(const float* qkv, const float* q_wei
 ATOM_EXPORT int atom_attention_prefill(const void* q, const void* k_cache, const void* v_cache, void* out,
                                        const int* cu_q, const int* ctx_lens, const int* block_tables, int max_blocks,
                                        const int* tiles, int num_tiles, int rows_per_tile, int tiled, int hq, int hkv,
-                                       int d, int page_size, float scale, int window, hipStream_t stream) {
+                                       int d, int page_size, float scale, int window, int chunk, float softcap,
+                                       hipStream_t stream) {
   if (int st = check_common(hq, hkv, d, page_size, max_blocks)) return st;
-  if (num_tiles < 0 || !tiles) return ATOM_BAD_SHAPE;
+  if (num_tiles < 0 || !tiles || window < 0 || chunk < 0 || softcap < 0.f) return ATOM_BAD_SHAPE;
+  if (softcap > 0.f && !(scale > 0.f)) return ATOM_UNSUPPORTED;
   if (num_tiles == 0) return ATOM_OK;
   AttnParams p{};
   p.q = (const bf16_t*)q; p.k_cache = (const bf16_t*)k_cache; p.v_cache = (const bf16_t*)v_cache;
   p.out = (bf16_t*)out; p.cu_q = cu_q; p.ctx_lens = ctx_lens; p.block_tables = block_tables; p.tiles = tiles;
   p.ws_o = nullptr; p.ws_ml = nullptr; p.max_blocks = max_blocks; p.hq = hq; p.hkv = hkv; p.page_size = page_size;
   p.window = window; p.seq_offset = 0; p.parts = 1; p.scale_log2 = scale * 1.4426950408889634f;
+  p.chunk = chunk;
+  if (softcap > 0.f) { p.cap_in = scale / softcap; p.cap_out = softcap / scale; }
   p.page_shift = page_shift_of(page_size);
   p.num_tiles = num_tiles;
   if (tiled) {   // tiles of atom_attention_prefill_tile_rows() tokens for the kernel with shared key tiles

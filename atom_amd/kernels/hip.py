@@ -564,7 +564,7 @@ class HipKernels:
             *self._sum_args(qkv), self._stream()))
         return q_out
 
-    def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None):
+    def _attention_mfma(self, q, k_cache, v_cache, out, meta, scale, window, parts=None, softcap=None, chunk=None):
         tokens, hq, d = q.shape
         _, hkv, page_size, _ = k_cache.shape
         self._check("cu_seqlens_q", meta.cu_seqlens_q, torch.int32, (meta.num_seqs + 1,))
@@ -589,11 +589,14 @@ class HipKernels:
             self._done("attention_prefill", self.lib.atom_attention_prefill(
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
                 _ptr(bt), bt.shape[1], _ptr(tiles), tiles.shape[0], rows, tiled, hq, hkv, d, page_size,
-                ctypes.c_float(scale), int(window or 0), self._stream()))
+                ctypes.c_float(scale), int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0),
+                self._stream()))
         seqs = meta.num_seqs - meta.num_prefill
         if seqs:
             if parts is None:
                 visible = min(meta.max_context_len, window) if window else meta.max_context_len
+                if chunk:
+                    visible = min(visible, chunk)
                 parts = self.decode_parts(seqs, hkv, visible)
             ws_o = ws_ml = None
             if parts > 1:
@@ -602,7 +605,8 @@ class HipKernels:
             self._done("attention_decode", self.lib.atom_attention_decode(
                 _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.cu_seqlens_q), _ptr(meta.context_lens),
                 _ptr(bt), bt.shape[1], meta.num_prefill, seqs, hq, hkv, d, page_size, ctypes.c_float(scale),
-                int(window or 0), parts, _ptr(ws_o), _ptr(ws_ml), self._stream()))
+                int(window or 0), int(chunk or 0), ctypes.c_float(softcap or 0.0), parts, _ptr(ws_o), _ptr(ws_ml),
+                self._stream()))
         return out
 
     def _prefill_in_halves(self, blocks: int, meta) -> bool:
@@ -704,9 +708,11 @@ class HipKernels:
         if meta.max_context_len > meta.block_tables.shape[1] * page_size:
             raise KernelError("attention: a context is longer than its block table can name")
         group = hq // hkv
-        if (dt == torch.bfloat16 and self.use_mfma_attention and not softcap and not chunk
+        if softcap and not scale > 0:
+            raise KernelError("attention: a cap on the scores needs a positive scale")
+        if (dt == torch.bfloat16 and self.use_mfma_attention
                 and self.lib.atom_attention_mfma_supports(d, page_size, group)):
-            return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts)
+            return self._attention_mfma(q, k_cache, v_cache, out, meta, scale, window, parts, softcap, chunk)
         self._done("paged_attention", self.lib.atom_paged_attention_generic(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(meta.token_seq), _ptr(meta.positions),
             _ptr(meta.block_tables), meta.block_tables.shape[1], self._code(q), tokens, hq, hkv, d, page_size,
