@@ -1221,12 +1221,17 @@ class HipKernels:
 
     # ------------------------------------------------------------------ the real-gated linear recurrence
 
+    #: tokens of a run of the gated recurrence's scan (the kernel's own constant)
+    RGLRU_RUN = 64
+
     def rglru_scan(self, u, gates, ra_bias, ri_bias, lam, proj, y_off: int, state, state_off: int, cu_seqlens_q,
-                   slot_of_seq, out, decay_scale: float):
+                   slot_of_seq, out, decay_scale: float, max_q_len: int | None = None):
         """``S <- a S + sqrt(1 - a^2) (i u)``, ``out = S * gelu_tanh(y)`` over each request's tokens, with
         ``r = sigmoid(gates[0] + ra_bias)``, ``i = sigmoid(gates[1] + ri_bias)``, ``a = exp(-decay_scale r
         softplus(lam))``.  ``u`` float32 [tokens, channels]; ``gates`` float32 [2, tokens, channels]; ``y`` the
-        ``channels`` columns of ``proj`` (float32) from ``y_off``; S at ``state_off`` of a slot's row of ``state``."""
+        ``channels`` columns of ``proj`` (float32) from ``y_off``; S at ``state_off`` of a slot's row of ``state``.
+        ``max_q_len``: the most tokens a request brings (an upper bound; default: all tokens); beyond a run's
+        length, runs of a request are scanned side by side."""
         tokens, channels = u.shape
         seqs = slot_of_seq.numel()
         self._check("recurrence input", u, torch.float32, (tokens, channels))
@@ -1242,10 +1247,16 @@ class HipKernels:
         self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
         self._check("recurrence out", out, (torch.float32, torch.bfloat16), (tokens, channels))
         gi = ctypes.c_void_p(gates.data_ptr() + 4 * tokens * channels)
+        longest = tokens if max_q_len is None else min(tokens, max_q_len)
+        ws, ws_floats = None, 0
+        if longest > self.RGLRU_RUN:
+            ws_floats = seqs * channels * (1 + 2 * -(-longest // self.RGLRU_RUN))
+            ws = self.workspace("rglru_runs", ws_floats)
         self._done("rglru_scan", self.lib.atom_rglru_scan(
             _ptr(u), _ptr(gates), gi, _ptr(ra_bias), _ptr(ri_bias), _ptr(lam), _ptr(proj), proj.shape[1], y_off,
             _ptr(state), ctypes.c_long(state.shape[1]), ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq),
-            seqs, _ptr(out), self._code(out), channels, ctypes.c_float(decay_scale), self._stream()))
+            seqs, _ptr(out), self._code(out), channels, ctypes.c_float(decay_scale), longest, _ptr(ws),
+            ctypes.c_long(ws_floats), self._stream()))
         return out
 
     # ------------------------------------------------------------------ attention whose values are its keys

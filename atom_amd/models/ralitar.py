@@ -31,7 +31,10 @@ def _mixer(cfg: RalitarConfig, layer: dict) -> PartChoice:
         return PartChoice("gated_delta", {
             "hidden_size": cfg.hidden_size, "num_heads": m["heads"], "num_kv_heads": m["kv_heads"],
             "head_dim": m["dim"], "value_dim": m["vdim"], "conv_taps": m["conv"], "norm_eps": cfg.norm_eps,
-            "decay": "channel", "decay_low_rank": True, "gate_low_rank": True, "gate_activation": "sigmoid"})
+            "decay": "channel", "decay_low_rank": True, "gate_low_rank": True, "gate_activation": "sigmoid",
+            # the inner sizes of the two low-rank projections are the checkpoint tensors' own; a configuration may
+            # name them for weights that are drawn, not loaded
+            "decay_rank": m.get("decay_rank"), "gate_rank": m.get("gate_rank")})
     rope = None
     rot = m.get("rot")
     if rot is not None and rot["dims"] > 0:

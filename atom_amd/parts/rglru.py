@@ -73,7 +73,8 @@ class RealGatedRecurrence(Mixer):
                            exact=True)
         out = torch.empty((T, c), dtype=x.dtype, device=x.device)
         ops.rglru_scan(u, gates, self.params["ra.bias"], self.params["ri.bias"], self.params["lam"], proj, c,
-                       cache.state, self.conv_floats, ctx.cu_seqlens_q, ctx.slot_of_seq, out, self.decay_scale)
+                       cache.state, self.conv_floats, ctx.cu_seqlens_q, ctx.slot_of_seq, out, self.decay_scale,
+                       max_q_len=ctx.max_q_len)
         return ops.linear(out, self.params["o.weight"], None, defer=True)
 
 

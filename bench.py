@@ -274,20 +274,57 @@ def lotorax_pair(size: str) -> tuple[dict, dict]:
     return loto, qwen
 
 
+# The Ralitar side has four layers (real-gated recurrence, delta rule with channel decay, chunked key-value attention,
+# recurrence again), each with a dense feed-forward and the token-side input, behind the pair embedding; the Qwen3
+# side four layers of the same width with a dense feed-forward of the same size.
+
+def ralitar_pair(size: str) -> tuple[dict, dict]:
+    width, heads, ff, vocab = {
+        "1k": (1024, 8, 2816, 32768),
+        "2k": (2048, 16, 5632, 32768),
+        "4k": (4096, 32, 11264, 65536),
+    }[size]
+    rot = {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    attn = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0,
+            "mask": {"size": 1024}, "rot": rot}
+    delta = {"heads": heads, "kv_heads": heads // 2, "dim": 128, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+    rec = {"width": width, "blocks": max(1, width // 256), "conv": 4}
+    dense = {"kind": "dense", "ff": ff}
+    rali = {"architecture": "Ralitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 7919}},
+            "token_side": {"dim": 256}, "max_position_embeddings": 40960,
+            "layers": [{"type": "rglru", "mixer": rec, "mlp": dense},
+                       {"type": "channel_delta", "mixer": delta, "mlp": dense},
+                       {"type": "attention", "mixer": attn, "mlp": dense},
+                       {"type": "rglru", "mixer": rec, "mlp": dense}]}
+    qwen = dict(QWEN3_8B, num_hidden_layers=4, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=max(1, heads // 4), intermediate_size=ff, vocab_size=vocab)
+    return rali, qwen
+
+
 def run_lotorax(args) -> dict:
     """Prefill and decode throughput of Lotorax and of Qwen3 at equal size, one engine after the other."""
+    return run_design(args, "lotorax", "Lotorax", lotorax_pair, args.lotorax)
+
+
+def run_ralitar(args) -> dict:
+    """Prefill and decode throughput of Ralitar and of Qwen3 at equal size, one engine after the other."""
+    return run_design(args, "ralitar", "Ralitar", ralitar_pair, args.ralitar)
+
+
+def run_design(args, key: str, design: str, pair, sizes: str) -> dict:
     import torch
 
     from atom_amd import LLMEngine, SamplingParams
     from atom_amd.config import model_config_from_dict
 
-    out = {"metric": "prefill tok/s and decode tok/s of the Lotorax design beside Qwen3 at equal size (bf16)",
+    out = {"metric": f"prefill tok/s and decode tok/s of the {design} design beside Qwen3 at equal size (bf16)",
            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
            "data": "synthetic: seeded uniform random token ids, seeded random N(0, 0.02) weights",
            "config": {"batch": args.batch, "context": args.context, "layers": 4}, "sizes": {}}
-    for size in args.lotorax.split(","):
+    for size in sizes.split(","):
         row = out["sizes"][size] = {}
-        for name, raw in zip(("lotorax", "qwen3"), lotorax_pair(size)):
+        for name, raw in zip((key, "qwen3"), pair(size)):
             max_len = max(4096, 2 * args.context)
             llm = LLMEngine(f"{name}-{size}-random", model_config=model_config_from_dict(raw), load_dummy="random",
                             seed=5, dtype="bf16", max_model_len=max_len, kv_cache_block_size=16,
@@ -312,9 +349,9 @@ def run_lotorax(args) -> dict:
                          "decode_tok_s": round(args.batch * args.steps / elapsed, 1)}
             print(f"[bench] {size} {name}: {row[name]}", file=sys.stderr, flush=True)
             release(llm)
-        row["prefill_ratio"] = round(row["lotorax"]["prefill_tok_s"] / row["qwen3"]["prefill_tok_s"], 3)
-        row["decode_ratio"] = round(row["lotorax"]["decode_tok_s"] / row["qwen3"]["decode_tok_s"], 3)
-    first = out["sizes"][args.lotorax.split(",")[0]]["lotorax"]
+        row["prefill_ratio"] = round(row[key]["prefill_tok_s"] / row["qwen3"]["prefill_tok_s"], 3)
+        row["decode_ratio"] = round(row[key]["decode_tok_s"] / row["qwen3"]["decode_tok_s"], 3)
+    first = out["sizes"][sizes.split(",")[0]][key]
     out.update(value=first["decode_tok_s"], ms_per_step=first["decode_ms_per_step"], higher_is_better=True,
                scaling="weak", vs_baseline=None)
     return out
@@ -568,6 +605,9 @@ def main() -> int:
     ap.add_argument("--lotorax", type=str, default="", metavar="SIZE[,SIZE]",
                     help="the Lotorax design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
                          "tokens and decode at --batch, four layers each")
+    ap.add_argument("--ralitar", type=str, default="", metavar="SIZE[,SIZE]",
+                    help="the Ralitar design beside Qwen3 at equal size (1k, 2k, 4k: the width): prefill of --context "
+                         "tokens and decode at --batch, four layers each")
     ap.add_argument("--budget", type=int, default=None,
                     help="the scheduler's token budget of a step (mixed: 512 + N by default, so that portions stay 512)")
     ap.add_argument("--temperature", type=float, default=0.0, help="of the decode steps' sampling (0: greedy)")
@@ -592,6 +632,9 @@ def main() -> int:
         return 0
     if args.lotorax:
         print(json.dumps(run_lotorax(args)), flush=True)
+        return 0
+    if args.ralitar:
+        print(json.dumps(run_ralitar(args)), flush=True)
         return 0
     args.shape = args.shape or "8b"
     line = run_shape(args)

@@ -345,7 +345,7 @@ class PlainKernels:
         return out
 
     def rglru_scan(self, u, gates, ra_bias, ri_bias, lam, proj, y_off, state, state_off, cu_seqlens_q, slot_of_seq, out,
-                   decay_scale):
+                   decay_scale, max_q_len=None):
         c = u.shape[1]
         sp = pr.softplus(lam.to(WIDE))
         for b in range(slot_of_seq.numel()):

@@ -145,12 +145,12 @@ def test_convolution_with_bias_and_without_activation(taps, channels):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("width,blocks", [(24, 3), (20, 1), (256, 4), (130, 2)])
-def test_gated_recurrence(dtype, width, blocks):
+@pytest.mark.parametrize("lens", [[37, 1, 5], [200, 1, 65], [64, 3, 129]])
+def test_gated_recurrence(dtype, width, blocks, lens):
     """The gates' small products and the scan against the plain mixer's inner loop, in two steps; lam reaches from
-    slow to fast decay."""
+    slow to fast decay.  Requests of more than 64 tokens are scanned in runs side by side."""
     ops = gpu_ops()
     part = width // blocks
-    lens = [37, 1, 5]
     T = sum(lens)
     u, ypre = rnd((T, width), 1), rnd((T, width), 2)
     ra, ri = rnd((blocks, part, part), 3, 2 / math.sqrt(part)).to(dtype), rnd((blocks, part, part), 4, 2 / math.sqrt(part)).to(dtype)
@@ -179,7 +179,8 @@ def test_gated_recurrence(dtype, width, blocks):
             ops.heads_gemm(ud, 0, width, part, wgt.to(DEV), gates, which * n * width, width, part, blocks, n, part, part,
                            exact=True)
         out = torch.empty((n, width), dtype=dtype, device=DEV)
-        ops.rglru_scan(ud, gates, rab.to(DEV), rib.to(DEV), lam.to(DEV), proj_rows.to(DEV), 3, state, 4, cu, sl, out, 8.0)
+        ops.rglru_scan(ud, gates, rab.to(DEV), rib.to(DEV), lam.to(DEV), proj_rows.to(DEV), 3, state, 4, cu, sl, out, 8.0,
+                       max_q_len=max(lens))
         return out, at
 
     out, at = run(u, proj, lens, [2, -1, 0])
