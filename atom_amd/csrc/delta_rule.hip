@@ -133,8 +133,9 @@ constexpr int kDPL = 16;   // entries of a column of S that one lane holds
 
 // qkv [T, channels] float32 after convolution and SiLU: q heads (kv_heads x dim) | k heads | v heads (heads x vdim).
 // ab [T, ld_ab] float32: the raw decay inputs at a_off and the raw beta inputs at b_off, one per head.
-// A column of S (dim entries) is spread over LPC adjacent lanes, entry i in lane i % LPC, so that a token costs each
-// lane 16 entries and two sums over the LPC lanes; the sums over a lane's entries run in four independent chains.
+// A column of S (dim entries) is spread over LPC adjacent lanes, entries 16 s .. 16 s + 15 in lane s of them (a lane's
+// part of a staged q, k or decay row is then 64 consecutive bytes of LDS, read 16 bytes at a time), so that a token costs
+// each lane 16 entries and two sums over the LPC lanes; the sums over a lane's entries run in four independent chains.
 //
 // CHANNEL: the decay is one number per head and key channel (row of S): dec holds heads x dim raw inputs a token at
 // a_off, dt_bias heads x dim entries, and a run's decays are staged like its q and k rows.
@@ -147,9 +148,9 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
                   const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads, int kv_heads, int dim,
                   int vdim) {
   constexpr int DMAX = kDPL * LPC;
-  __shared__ float qs[kRun][DMAX];
-  __shared__ float ks[kRun][DMAX];
-  __shared__ float gv[CHANNEL ? kRun : 1][DMAX];   // CHANNEL: a run's decays per key channel
+  __shared__ __attribute__((aligned(16))) float qs[kRun][DMAX];
+  __shared__ __attribute__((aligned(16))) float ks[kRun][DMAX];
+  __shared__ __attribute__((aligned(16))) float gv[CHANNEL ? kRun : 1][DMAX];   // CHANNEL: a run's decays per key channel
   __shared__ float gs[kRun], bs[kRun];
   const int head = blockIdx.x, seq = blockIdx.y;
   const int tid = threadIdx.x;
@@ -168,7 +169,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   float S[kDPL];
 #pragma unroll
   for (int j = 0; j < kDPL; ++j) {
-    const int i = j * LPC + sub;
+    const int i = sub * kDPL + j;
     S[j] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
   }
   const float decay_rate = -expf(a_log[head]);
@@ -255,10 +256,12 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     // a token's k and q entries are read from LDS one token ahead of their use, so that the chain below never
     // waits for them
     float kc[kDPL], qc[kDPL], kn[kDPL], qn[kDPL];
+    float gc[CHANNEL ? kDPL : 1], gn[CHANNEL ? kDPL : 1];
 #pragma unroll
     for (int e = 0; e < kDPL; ++e) {
-      kc[e] = ks[0][e * LPC + sub];
-      qc[e] = qs[0][e * LPC + sub];
+      kc[e] = ks[0][sub * kDPL + e];
+      qc[e] = qs[0][sub * kDPL + e];
+      if constexpr (CHANNEL) gc[e] = gv[0][sub * kDPL + e];
     }
 #pragma unroll
     for (int j = 0; j < kRun; ++j) {
@@ -266,16 +269,13 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       const float g = CHANNEL ? 1.f : gs[j];
       const float beta = bs[j];
       const float v = vv[j];
-      float gc[kDPL];
-      if constexpr (CHANNEL) {
-#pragma unroll
-        for (int e = 0; e < kDPL; ++e) gc[e] = gv[j][e * LPC + sub];
-      }
+
       if (j + 1 < kRun) {
 #pragma unroll
         for (int e = 0; e < kDPL; ++e) {
-          kn[e] = ks[j + 1][e * LPC + sub];
-          qn[e] = qs[j + 1][e * LPC + sub];
+          kn[e] = ks[j + 1][sub * kDPL + e];
+          qn[e] = qs[j + 1][sub * kDPL + e];
+          if constexpr (CHANNEL) gn[e] = gv[j + 1][sub * kDPL + e];
         }
       }
       float part[4] = {0.f, 0.f, 0.f, 0.f};
@@ -298,13 +298,14 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       for (int e = 0; e < kDPL; ++e) {
         kc[e] = kn[e];
         qc[e] = qn[e];
+        if constexpr (CHANNEL) gc[e] = gn[e];
       }
       }
     }
   }
 #pragma unroll
   for (int j = 0; j < kDPL; ++j) {
-    const int i = j * LPC + sub;
+    const int i = sub * kDPL + j;
     if (live && i < dim) sp[(size_t)i * vdim + col] = S[j];
   }
 }
