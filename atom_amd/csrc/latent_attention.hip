@@ -158,6 +158,43 @@ heads_gemm_kernel(const TX* __restrict__ x, long ldx, long hsx, const TW* __rest
   }
 }
 
+// The same product for few rows (single tokens): a wave owns one output column of one head, reads its row of w once,
+// 64 entries a step with all loads of a step independent, and multiplies it with up to 8 rows of x; the 64 partial sums
+// of a row are added across the wave.  The tile kernel above walks K in steps of 16 with a barrier and a wait for
+// memory in each, which for 8 rows is all it does.
+constexpr int kHFewRows = 8;
+
+template <typename TX, typename TW, typename TY>
+__global__ void __launch_bounds__(256)
+heads_rows_kernel(const TX* __restrict__ x, long ldx, long hsx, const TW* __restrict__ w, TY* __restrict__ y, long ldy,
+                  long hsy, const float* __restrict__ gate, long ldg, int m, int n, int k, float alpha) {
+  const int lane = threadIdx.x % kWave;
+  const int col = blockIdx.x * (256 / kWave) + threadIdx.x / kWave;
+  const int h = blockIdx.y;
+  if (col >= n) return;
+  const TX* xh = x + (size_t)h * hsx;
+  const TW* wr = w + ((size_t)h * n + col) * k;
+  float acc[kHFewRows];
+#pragma unroll
+  for (int r = 0; r < kHFewRows; ++r) acc[r] = 0.f;
+  for (int kk = lane; kk < k; kk += kWave) {
+    const float wv = to_f32(wr[kk]);
+#pragma unroll
+    for (int r = 0; r < kHFewRows; ++r)
+      if (r < m) acc[r] = fmaf(to_f32(xh[(size_t)r * ldx + kk]), wv, acc[r]);
+  }
+#pragma unroll
+  for (int r = 0; r < kHFewRows; ++r) {
+    if (r >= m) continue;
+    const float total = wave_sum(acc[r]);
+    if (lane == 0) {
+      float f = alpha;
+      if (gate) f *= 1.f / (1.f + expf(-gate[(size_t)r * ldg + h]));
+      y[(size_t)r * ldy + (size_t)h * hsy + col] = from_f32<TY>(total * f);
+    }
+  }
+}
+
 ATOM_EXPORT int atom_heads_gemm(const void* x, int x_dtype, long ldx, long hsx, const void* w, int w_dtype, void* y,
                                 int y_dtype, long ldy, long hsy, const float* gate, long ldg, int heads, int m, int n,
                                 int k, float alpha, hipStream_t stream) {
@@ -165,11 +202,19 @@ ATOM_EXPORT int atom_heads_gemm(const void* x, int x_dtype, long ldx, long hsx, 
   if (x == nullptr || w == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
   if ((unsigned)x_dtype > 1u || (unsigned)w_dtype > 1u || (unsigned)y_dtype > 1u) return ATOM_BAD_DTYPE;
   if (m == 0) return ATOM_OK;
+  const bool few = m <= kHFewRows;
   dim3 grid((n + kHTile - 1) / kHTile, (m + kHTile - 1) / kHTile, heads), block(256);
+  if (few) grid = dim3((n + 3) / 4, heads, 1);
   if (grid.y > 65535) return ATOM_TOO_LARGE;
-#define LAUNCH(TX, TW, TY)                                                                                        \
-  hipLaunchKernelGGL((heads_gemm_kernel<TX, TW, TY>), grid, block, 0, stream, (const TX*)x, ldx, hsx, (const TW*)w, \
-                     (TY*)y, ldy, hsy, gate, ldg, m, n, k, alpha)
+#define LAUNCH(TX, TW, TY)                                                                                          \
+  do {                                                                                                              \
+    if (few)                                                                                                        \
+      hipLaunchKernelGGL((heads_rows_kernel<TX, TW, TY>), grid, block, 0, stream, (const TX*)x, ldx, hsx, (const TW*)w, \
+                         (TY*)y, ldy, hsy, gate, ldg, m, n, k, alpha);                                              \
+    else                                                                                                            \
+      hipLaunchKernelGGL((heads_gemm_kernel<TX, TW, TY>), grid, block, 0, stream, (const TX*)x, ldx, hsx, (const TW*)w, \
+                         (TY*)y, ldy, hsy, gate, ldg, m, n, k, alpha);                                              \
+  } while (0)
   switch (x_dtype * 4 + w_dtype * 2 + y_dtype) {
     case 0: LAUNCH(float, float, float); break;
     case 1: LAUNCH(float, float, bf16_t); break;
