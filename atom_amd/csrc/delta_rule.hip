@@ -12,11 +12,14 @@
 //
 //   conv_silu_state   one thread per (request, channel, run of 64 tokens); optionally a bias per channel, and SiLU or
 //                     no activation
+//   delta_prepare     a block per token: unit q and k, decays from their raw inputs, in place
 //   delta_rule        blocks per (request, head, group of columns); a column of S (over dim) sits in the registers of up
 //                     to 16 adjacent lanes, so the columns never meet; q, k and the gates of a run of tokens are
 //                     staged in LDS
 //   delta_out         o / rms(o) * w * silu(gate) (or sigmoid(gate)), rounded to the serving type
 #include "common.h"
+
+#include <type_traits>
 
 constexpr int kMaxTaps = 16;
 
@@ -128,6 +131,33 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// What does not depend on the state is done for all tokens side by side, in place, before the recurrence walks them:
+// q and k become unit vectors per head (q also times dim^-1/2), and the raw decay inputs become the decays
+// exp(-exp(A_log) softplus(a + dt_bias)), one per head or one per head and key channel.  A block per token.
+__global__ void __launch_bounds__(256)
+delta_prepare_kernel(float* __restrict__ qkv, int channels, float* __restrict__ dec, int ld_dec, int a_off,
+                     const float* __restrict__ a_log, const float* __restrict__ dt_bias, int heads, int kv_heads, int dim,
+                     int per_head) {
+  const size_t t = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const float q_scale = 1.f / sqrtf((float)dim);
+  for (int row = wave; row < 2 * kv_heads; row += 256 / kWave) {
+    float* r = qkv + t * channels + (size_t)row * dim;
+    float ss = 0.f;
+    for (int i = lane; i < dim; i += kWave) ss += r[i] * r[i];
+    ss = wave_sum(ss);
+    const float f = (row < kv_heads ? q_scale : 1.f) / sqrtf(ss + 1e-6f);
+    for (int i = lane; i < dim; i += kWave) r[i] *= f;
+  }
+  float* d = dec + t * ld_dec + a_off;
+  const int wide = heads * per_head;
+  for (int i = threadIdx.x; i < wide; i += blockDim.x) {
+    const float z = d[i] + dt_bias[i];
+    const float sp_z = z > 20.f ? z : log1pf(expf(z));
+    d[i] = expf(-expf(a_log[i / per_head]) * sp_z);
+  }
+}
+
 constexpr int kRun = 16;   // tokens whose q, k and gates are staged at once
 constexpr int kDPL = 16;   // entries of a column of S that one lane holds
 
@@ -143,7 +173,7 @@ template <int LPC, bool CHANNEL>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab,
                   const float* __restrict__ dec, int ld_dec, int a_off,
-                  int b_off, const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                  int b_off,
                   float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
                   const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads, int kv_heads, int dim,
                   int vdim) {
@@ -172,11 +202,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     const int i = sub * kDPL + j;
     S[j] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
   }
-  const float decay_rate = -expf(a_log[head]);
-  const float bias = CHANNEL ? 0.f : dt_bias[head];
-  const float q_scale = 1.f / sqrtf((float)dim);
   const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
-  const int wave = tid / kWave, lane = tid % kWave;
   // A run's q and k rows, its values of this column and its gates travel memory -> registers -> LDS; the registers
   // are filled for the next run while this run's tokens are worked through, so that no load is waited for inside
   // the chain of tokens.
@@ -224,33 +250,16 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       for (int it = 0; it < G_ITEMS; ++it) {
         const int idx = tid + it * 256;
         const int j = idx / DMAX, i = idx % DMAX;
-        const float z = g_raw[it] + (i < dim ? dt_bias[head * dim + i] : 0.f);
-        const float sp_z = z > 20.f ? z : log1pf(expf(z));
-        gv[j][i] = expf(decay_rate * sp_z);
+        gv[j][i] = g_raw[it];
       }
     }
     if (tid < n) {
-      if constexpr (!CHANNEL) {
-        const float z = a_next + bias;
-        const float sp_z = z > 20.f ? z : log1pf(expf(z));
-        gs[tid] = expf(decay_rate * sp_z);
-      }
+      if constexpr (!CHANNEL) gs[tid] = a_next;
       bs[tid] = 1.f / (1.f + expf(-b_next));
     }
     float vv[kRun];
 #pragma unroll
     for (int j = 0; j < kRun; ++j) vv[j] = v_next[j];
-    __syncthreads();
-    // unit vectors: a wave per (token, q or k), in place
-    for (int item = wave; item < 2 * n; item += 4) {
-      const int j = item >> 1, is_k = item & 1;
-      float* dst = is_k ? ks[j] : qs[j];
-      float ss = 0.f;
-      for (int i = lane; i < DMAX; i += kWave) ss += dst[i] * dst[i];
-      ss = wave_sum(ss);
-      const float f = (is_k ? 1.f : q_scale) / sqrtf(ss + 1e-6f);
-      for (int i = lane; i < DMAX; i += kWave) dst[i] *= f;
-    }
     __syncthreads();
     if (t0 + kRun < end) load_run(t0 + kRun);
     // a token's k and q entries are read from LDS one token ahead of their use, so that the chain below never
@@ -263,9 +272,12 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       qc[e] = qs[0][sub * kDPL + e];
       if constexpr (CHANNEL) gc[e] = gv[0][sub * kDPL + e];
     }
+    // A whole run is walked without a test per token: the registers that hold the next token's entries then simply
+    // become the current ones, with no copies (a test per token makes every hand-over a set of moves).
+    auto walk = [&](auto whole) {
 #pragma unroll
     for (int j = 0; j < kRun; ++j) {
-      if (j < n) {
+      if (decltype(whole)::value || j < n) {
       const float g = CHANNEL ? 1.f : gs[j];
       const float beta = bs[j];
       const float v = vv[j];
@@ -302,6 +314,9 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       }
       }
     }
+    };
+    if (n == kRun) walk(std::true_type{});
+    else walk(std::false_type{});
   }
 #pragma unroll
   for (int j = 0; j < kDPL; ++j) {
@@ -310,7 +325,8 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
   }
 }
 
-ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab, int ld_ab, const float* dec, int ld_dec,
+// qkv and the decay inputs are changed in place (see delta_prepare_kernel); tokens is the number of their rows.
+ATOM_EXPORT int atom_delta_rule(float* qkv, int tokens, int channels, const float* ab, int ld_ab, float* dec, int ld_dec,
                                 int a_off, int b_off, int per_channel,
                                 const float* a_log, const float* dt_bias, float* state, long slot_stride,
                                 long state_off, const int* cu_seqlens, const int* slot_of_seq, int num_seqs, float* out,
@@ -322,8 +338,10 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
   if (ab == nullptr || dec == nullptr) return ATOM_BAD_SHAPE;
   if (state_off < 0 || slot_stride < state_off + (long)heads * dim * vdim) return ATOM_BAD_SHAPE;
   if (dim > 256) return ATOM_TOO_LARGE;
-  if (num_seqs == 0) return ATOM_OK;
+  if (num_seqs == 0 || tokens <= 0) return ATOM_OK;
   if (num_seqs > 65535 || heads > 65535) return ATOM_TOO_LARGE;
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(tokens), dim3(256), 0, stream, qkv, channels, dec, ld_dec, a_off, a_log,
+                     dt_bias, heads, kv_heads, dim, per_channel ? dim : 1);
   int lpc = 1;
   while (lpc * kDPL < dim) lpc *= 2;
   const int cols = 256 / lpc;
@@ -331,8 +349,7 @@ ATOM_EXPORT int atom_delta_rule(const float* qkv, int channels, const float* ab,
   if (grid.z > 65535) return ATOM_TOO_LARGE;
 #define LAUNCH_AS(L, C)                                                                                          \
   hipLaunchKernelGGL((delta_rule_kernel<L, C>), grid, block, 0, stream, qkv, channels, ab, ld_ab, dec, ld_dec, a_off, \
-                     b_off, a_log, dt_bias, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads,     \
-                     kv_heads, dim, vdim)
+                     b_off, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim, vdim)
 #define LAUNCH(L)                  \
   do {                             \
     if (per_channel) {             \

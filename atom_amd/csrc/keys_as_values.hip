@@ -6,7 +6,7 @@
 //   q goes to q_out [T, H, D]; the normed, rotated k to the key pages [pages, G, page, D]; k as projected to
 //   the value pages [pages, G, D, page].
 //
-// A block per token.  sigmoid_gate multiplies the heads' outputs by the sigmoid of the gate's columns of the product.
+// A block per token; a token's angles are formed once and shared by its heads through LDS.  sigmoid_gate multiplies the heads' outputs by the sigmoid of the gate's columns of the product.
 #include "common.h"
 
 __device__ __forceinline__ void turn_angle(int position, double freq, float* c, float* s) {
@@ -23,6 +23,7 @@ keys_as_values_write_kernel(const float* __restrict__ proj, int ld, T* __restric
                             const double* __restrict__ freq, int rot_dims, const int* __restrict__ positions,
                             const int* __restrict__ slots, int H, int G, int D, int page_size, float eps) {
   __shared__ float scratch[16];
+  extern __shared__ float turn[];   // cosines of the token's rot_dims / 2 angles, then their sines
   const int t = blockIdx.x;
   const int Q = H * D, K = G * D;
   const float* qr = proj + (size_t)t * ld;
@@ -39,6 +40,9 @@ keys_as_values_write_kernel(const float* __restrict__ proj, int ld, T* __restric
     inv_k = 1.f / sqrtf(block_sum(ss, scratch) / (float)K + eps);
   }
   const int pos = rot_dims > 0 ? positions[t] : 0;
+  const int pairs = rot_dims / 2;
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) turn_angle(pos, freq[i], &turn[i], &turn[pairs + i]);
+  __syncthreads();
   const int slot = slots != nullptr ? slots[t] : -1;
   const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
   for (int e = threadIdx.x; e < Q + K; e += blockDim.x) {
@@ -52,8 +56,7 @@ keys_as_values_write_kernel(const float* __restrict__ proj, int ld, T* __restric
     if (i < rot_dims) {
       const int other = j - i + (i ^ 1);
       const float p = row[other] * (w != nullptr ? inv * w[other] : 1.f);
-      float c, s;
-      turn_angle(pos, freq[i >> 1], &c, &s);
+      const float c = turn[i >> 1], s = turn[pairs + (i >> 1)];
       v = (i & 1) ? v * c + p * s : v * c - p * s;
     }
     if (!is_k) {
@@ -75,7 +78,8 @@ ATOM_EXPORT int atom_keys_as_values_write(const float* proj, int ld, void* q_out
   if (proj == nullptr || q_out == nullptr) return ATOM_BAD_SHAPE;
   if (slots != nullptr && (k_cache == nullptr || v_cache == nullptr)) return ATOM_BAD_SHAPE;
   if (tokens == 0) return ATOM_OK;
-  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((keys_as_values_write_kernel<T>), dim3(tokens), dim3(256), 0, stream, proj,
+  const size_t smem = (size_t)(rot_dims > 0 ? rot_dims : 1) * sizeof(float);
+  ATOM_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((keys_as_values_write_kernel<T>), dim3(tokens), dim3(256), smem, stream, proj,
                                                  ld, (T*)q_out, (T*)k_cache, (T*)v_cache, qw, kw, freq, rot_dims, positions,
                                                  slots, H, G, D, page_size, eps));
   return launch_status();

@@ -1109,7 +1109,8 @@ class HipKernels:
         ``b_off`` and, unless ``decay`` (float32 [tokens, *]) holds them, the raw decay inputs at ``a_off``: one
         per head, or with ``per_channel`` one per head and key channel (``dt_bias`` likewise); the heads' matrices
         [heads, dim, vdim] start at ``state_off`` of a slot's row of ``state``.  ``out`` float32 [tokens, heads,
-        vdim]."""
+        vdim].  ``qkv`` and the decay inputs are used up: q and k are made unit vectors and the raw decay inputs
+        become the decays, in place, for all tokens side by side before the recurrence walks them."""
         tokens, channels = qkv.shape
         seqs = slot_of_seq.numel()
         decay = gates if decay is None else decay
@@ -1126,7 +1127,7 @@ class HipKernels:
         self._check("slot_of_seq", slot_of_seq, torch.int32, (seqs,))
         self._check("delta out", out, torch.float32, (tokens, heads, vdim))
         self._done("delta_rule", self.lib.atom_delta_rule(
-            _ptr(qkv), channels, _ptr(gates), gates.shape[1], _ptr(decay), decay.shape[1], a_off, b_off,
+            _ptr(qkv), tokens, channels, _ptr(gates), gates.shape[1], _ptr(decay), decay.shape[1], a_off, b_off,
             int(bool(per_channel)), _ptr(a_log), _ptr(dt_bias), _ptr(state),
             ctypes.c_long(state.shape[1]), ctypes.c_long(state_off), _ptr(cu_seqlens_q), _ptr(slot_of_seq), seqs,
             _ptr(out), heads, kv_heads, dim, vdim, self._stream()))
