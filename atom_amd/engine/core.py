@@ -50,7 +50,7 @@ class EngineCore:
         self.dtype = dtype
         self.plan = plan
         # the prefix cache needs every mixer's memory to be pages that keep all that earlier tokens left
-        needs = [model.blocks[run.layer].mixer.cache_need() for run in model.order]
+        needs = [model.blocks[run.layer].mixer.cache_need() for run in model.order] + [model.embedding.cache_need()]
         self.prefix_caching = bool(prefix_caching and plan.groups and all(
             kind_of(n).keeps_every_token(n) for n in needs if n is not None))
         self.manager = CacheManager(plan.groups, max_num_seqs, prefix_caching=self.prefix_caching)

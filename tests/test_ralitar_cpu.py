@@ -214,3 +214,20 @@ def test_greedy_generation_through_the_engine():
             assert token == int(rt.oracle("V", tokens)[-1].argmax())
             tokens.append(token)
     assert all(p.num_free == p.num_pages for p in llm.core.manager.pools)
+
+
+def test_prefix_cache_stays_off_where_the_embedding_keeps_a_token():
+    """A request that took over cached pages would start without its previous token: the prefix cache is on only
+    where nothing but pages is kept, and the pair embedding keeps a token per request."""
+    import torch
+    from atom_amd.engine.core import build_core
+
+    raw = copy.deepcopy(rt.RALI_W)
+    raw["layers"] = [layer for layer in raw["layers"] if layer["type"] == "attention"]
+    for layer in raw["layers"]:
+        layer["mixer"].pop("mask")
+    bare = build_model(model_config_from_dict(raw))
+    assert build_core(bare, PlainKernels(), dtype=torch.float32, device="cpu", num_pages=4, prefix_caching=True).prefix_caching
+    raw["embedding"] = {"bigram": {"buckets": 7, "mul_prev": 3, "mul_cur": 5}}
+    paired = build_model(model_config_from_dict(raw))
+    assert not build_core(paired, PlainKernels(), dtype=torch.float32, device="cpu", num_pages=4, prefix_caching=True).prefix_caching
