@@ -20,7 +20,7 @@ import zlib
 import torch
 
 # inner sizes of the delta rule's low-rank projections: a tensor's shape says them, the configuration does not
-RANKS = {"U": {"a1": 6, "g1": 10}, "V": {"a1": 9, "g1": 4}, "W": {"a1": 16, "g1": 24}}
+RANKS = {"U": {"a1": 6, "g1": 10}, "V": {"a1": 9, "g1": 4}, "W": {"a1": 16, "g1": 24}, "X": {"a1": 40, "g1": 24}}
 
 
 def _rglru(width, blocks, conv):
@@ -86,8 +86,21 @@ RALI_W = {
     ],
 }
 
-CONFIGS = {"U": RALI_U, "V": RALI_V, "W": RALI_W}
-SEEDS = {"U": 5, "V": 13, "W": 31}
+# X: wide enough that prompts of 5, 40, 130 and 300 tokens reach every kernel the engine has for matrix products
+# (few rows, up to 64, up to 256, the library's), with widths that are not powers of two
+RALI_X = {
+    "architecture": "Ralitar", "vocab": 1000, "width": 384, "norm": {"eps": 1e-6},
+    "embedding": {"bigram": {"buckets": 509, "mul_prev": 65537, "mul_cur": 257}}, "token_side": {"dim": 24},
+    "layers": [
+        {"type": "attention", "mixer": _attn(6, 3, 64, 96, 0.125, softcap=30.0, rot={"base": 10000.0, "dims": 16, "scaling": BANDS}),
+         "mlp": _dense(1056)},
+        {"type": "channel_delta", "mixer": _delta(6, 3, 64, 32, 4), "mlp": _dense(1056)},
+        {"type": "rglru", "mixer": _rglru(448, 7, 4), "mlp": _dense(1056)},
+    ],
+}
+
+CONFIGS = {"U": RALI_U, "V": RALI_V, "W": RALI_W, "X": RALI_X}
+SEEDS = {"U": 5, "V": 13, "W": 31, "X": 43}
 
 
 def _draw(name: str, shape, seed: int) -> torch.Tensor:

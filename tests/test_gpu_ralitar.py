@@ -406,7 +406,8 @@ def test_a_key_that_stands_out_is_seen_inside_its_chunk_only(dtype, D, page, chu
 
 # ------------------------------------------------------------------ the engine
 
-LENGTHS = {"U": [1, 7, 33, 150, 64, 300], "V": [2, 19, 45, 260, 128], "W": [3, 40, 17, 270, 96, 161]}
+LENGTHS = {"U": [1, 7, 33, 150, 64, 300], "V": [2, 19, 45, 260, 128], "W": [3, 40, 17, 270, 96, 161],
+           "X": [5, 40, 130, 300]}
 # float32: every position against the largest logit of its request; where the plain implementation in float32 is
 # itself further from float64 than that (a token whose sublayer output is small before its norm), four times its
 # own distance is allowed
@@ -453,6 +454,19 @@ def test_cuts_match_plain(which, cut, dtype):
     assert all(pool.num_free == pool.num_pages for pool in core.manager.pools)
     if cut == "tail":
         assert core.graphs is not None and core.graphs.replays >= 32, "single tokens replay captured graphs"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "mixed"])
+def test_wider_model_reaches_every_product_kernel(cut, dtype):
+    """Prompts of 5, 40, 130 and 300 tokens on a model of width 384: products of few rows, of up to 64, of up to 256
+    and the library's, with float32 outputs and biases, all against the plain implementation."""
+    requests = _requests("X")
+    steps = getattr(replay, cut)(requests)
+    pages = -(-replay.peak_tokens(steps, 16) // 16)
+    core = rt.core("X", dtype, gpu_ops(), DEV, num_pages=pages, page_size=16, graph_sizes=[1, 2, 4] if cut != "whole" else None)
+    results = replay.run_in_process(core, steps)
+    _check(steps, results, requests, "X", dtype, f"X/{cut}/{dtype}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
