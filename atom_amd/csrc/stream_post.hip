@@ -41,15 +41,107 @@ rmsnorm_post_kernel(const TX* __restrict__ x, const float* __restrict__ weight, 
   }
 }
 
+// The same for widths that are a multiple of 4 and at most 4 * 256 * VPT: a thread keeps VPT groups of 4 consecutive
+// elements in registers, every load of a row is issued before the sum of squares is formed (16-byte accesses of the
+// stream and the weight, 8- or 16-byte ones of x), and nothing goes through LDS but the reduction.
+template <typename T>
+struct Quad;
+template <>
+struct Quad<float> {
+  float4 v;
+  __device__ __forceinline__ void get(float* f) const { f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w; }
+  __device__ __forceinline__ void set(const float* f) { v = make_float4(f[0], f[1], f[2], f[3]); }
+};
+template <>
+struct alignas(8) Quad<bf16_t> {
+  bf16_t v[4];
+  __device__ __forceinline__ void get(float* f) const {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = static_cast<float>(v[e]);
+  }
+  __device__ __forceinline__ void set(const float* f) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = static_cast<bf16_t>(f[e]);
+  }
+};
+
+template <typename TX, typename TO, int VPT>
+__global__ void __launch_bounds__(256)
+rmsnorm_post_vec_kernel(const TX* __restrict__ x, const float* __restrict__ weight, float eps, float* __restrict__ stream,
+                        TO* __restrict__ out, int width) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  const TX* xr = x + row * width;
+  float* sr = stream + row * width;
+  Quad<TX> xq[VPT];
+  float4 sq[VPT], wq[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * 256) * 4;
+    if (i < width) {
+      xq[j] = *reinterpret_cast<const Quad<TX>*>(xr + i);
+      sq[j] = *reinterpret_cast<const float4*>(sr + i);
+      wq[j] = *reinterpret_cast<const float4*>(weight + i);
+    }
+  }
+  float vals[VPT][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * 256) * 4;
+    if (i < width) {
+      xq[j].get(vals[j]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += vals[j][e] * vals[j][e];
+    }
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int i = (threadIdx.x + j * 256) * 4;
+    if (i < width) {
+      float s4[4] = {sq[j].x, sq[j].y, sq[j].z, sq[j].w};
+      const float w4[4] = {wq[j].x, wq[j].y, wq[j].z, wq[j].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s4[e] += vals[j][e] * inv * w4[e];
+      *reinterpret_cast<float4*>(sr + i) = make_float4(s4[0], s4[1], s4[2], s4[3]);
+      if (out != nullptr) {
+        Quad<TO> o;
+        o.set(s4);
+        *reinterpret_cast<Quad<TO>*>(out + row * width + i) = o;
+      }
+    }
+  }
+}
+
 ATOM_EXPORT int atom_rmsnorm_post(const void* x, int x_dtype, const float* weight, float eps, float* stream, void* out,
                                   int out_dtype, int rows, int width, hipStream_t stream_handle) {
   if (rows < 0 || width <= 0 || x == nullptr || weight == nullptr || stream == nullptr) return ATOM_BAD_SHAPE;
   if (width > 32768) return ATOM_TOO_LARGE;
   if (rows == 0) return ATOM_OK;
   const size_t smem = (size_t)(width + 16) * sizeof(float);
-#define LAUNCH(TX, TO)                                                                                             \
-  hipLaunchKernelGGL((rmsnorm_post_kernel<TX, TO>), dim3(rows), dim3(256), smem, stream_handle, (const TX*)x, weight, \
-                     eps, stream, (TO*)out, width)
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)stream % 16 == 0) && ((uintptr_t)weight % 16 == 0) &&
+                       (out == nullptr || (uintptr_t)out % 16 == 0);
+  const int vpt = (width % 4 == 0 && aligned) ? (width + 1023) / 1024 : 0;   // groups of 4 a thread; 0: the general kernel
+#define LAUNCH(TX, TO)                                                                                               \
+  do {                                                                                                               \
+    if (vpt == 1)                                                                                                    \
+      hipLaunchKernelGGL((rmsnorm_post_vec_kernel<TX, TO, 1>), dim3(rows), dim3(256), 0, stream_handle, (const TX*)x, \
+                         weight, eps, stream, (TO*)out, width);                                                      \
+    else if (vpt == 2)                                                                                               \
+      hipLaunchKernelGGL((rmsnorm_post_vec_kernel<TX, TO, 2>), dim3(rows), dim3(256), 0, stream_handle, (const TX*)x, \
+                         weight, eps, stream, (TO*)out, width);                                                      \
+    else if (vpt >= 3 && vpt <= 4)                                                                                   \
+      hipLaunchKernelGGL((rmsnorm_post_vec_kernel<TX, TO, 4>), dim3(rows), dim3(256), 0, stream_handle, (const TX*)x, \
+                         weight, eps, stream, (TO*)out, width);                                                      \
+    else if (vpt >= 5 && vpt <= 8)                                                                                   \
+      hipLaunchKernelGGL((rmsnorm_post_vec_kernel<TX, TO, 8>), dim3(rows), dim3(256), 0, stream_handle, (const TX*)x, \
+                         weight, eps, stream, (TO*)out, width);                                                      \
+    else                                                                                                             \
+      hipLaunchKernelGGL((rmsnorm_post_kernel<TX, TO>), dim3(rows), dim3(256), smem, stream_handle, (const TX*)x,    \
+                         weight, eps, stream, (TO*)out, width);                                                      \
+  } while (0)
   const bool out_bf16 = out != nullptr && out_dtype == ATOM_BF16;
   if (out != nullptr && out_dtype != ATOM_BF16 && out_dtype != ATOM_F32) return ATOM_BAD_DTYPE;
   if (x_dtype == ATOM_F32) {

@@ -40,7 +40,7 @@ def i32(values):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,n", [(40, 7), (333, 5), (4096, 3), (64, 300)])
+@pytest.mark.parametrize("width,n", [(40, 7), (333, 5), (4096, 3), (64, 300), (2048, 9), (1500, 4), (6148, 3), (8200, 2)])
 def test_normed_summands_join_the_stream(dtype, width, n):
     ops = gpu_ops()
     stream = rnd((n, width), 1, 2.0)
