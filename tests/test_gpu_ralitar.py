@@ -247,6 +247,79 @@ def test_delta_rule_with_a_decay_per_channel(heads, kv_heads, dim, vdim):
         close(part, plain(list(range(21)), zero)[0][lo:hi], torch.float32, f"rows {lo}-{hi}")
 
 
+def test_far_tokens_stay_in_the_recurrent_states():
+    """With decays close to 1, what the first token wrote is read 1,400 tokens later: by the gated recurrence (whole,
+    and in three steps that hand the state on) and by the delta rule, whose later tokens write next to nothing.
+    Without the first token the same read-out is far smaller, so a state lost on the way would show."""
+    ops = gpu_ops()
+    T, width = 1400, 24
+    lam = torch.full((width,), -9.0)                       # a = exp(-8 r softplus(-9)): about 0.9995 a token
+    u = rnd((T, width), 1, 0.001)
+    u[0] = 5.0
+    ypre = torch.ones(T, width)
+    zeros = torch.zeros(1, width)
+    ident = torch.zeros(1, width, width)
+    proj = torch.cat((torch.zeros(T, 3), ypre), dim=1)
+
+    def scan(u_rows, cuts):
+        state = torch.zeros((1, 4 + width), dtype=torch.float32, device=DEV)
+        outs, at = [], 0
+        for n in cuts:
+            rows = u_rows[at:at + n].contiguous().to(DEV)
+            gates = torch.zeros((2, n, width), dtype=torch.float32, device=DEV)
+            out = torch.empty((n, width), dtype=torch.float32, device=DEV)
+            ops.rglru_scan(rows, gates, zeros.to(DEV), zeros.to(DEV), lam.to(DEV), proj[at:at + n].contiguous().to(DEV), 3,
+                           state, 4, i32([0, n]), i32([0]), out, 8.0, max_q_len=n)
+            outs.append(out.cpu())
+            at += n
+        return torch.cat(outs)
+
+    S = torch.zeros(width, dtype=torch.float64)
+    a = torch.exp(-8.0 * 0.5 * pr.softplus(lam.double()))
+    want = torch.zeros(T, width, dtype=torch.float64)
+    for t in range(T):
+        S = a * S + torch.sqrt(1 - a * a) * (0.5 * u[t].double())
+        want[t] = S * pr.gelu_tanh(ypre[t].double())
+    whole = scan(u, [T])
+    close(whole, want, torch.float32, "whole")
+    close(scan(u, [700, 1, 699]), want, torch.float32, "in three steps")
+    without = u.clone()
+    without[0] = 0
+    assert float(whole[-1].abs().min()) > 20 * float(scan(without, [T])[-1].abs().max())
+
+    # the delta rule: token 0 writes v0 under k0; later tokens have beta of about e^-20 and decays of about 1
+    H = G = 1
+    D, V = 16, 8
+    qkv = rnd((T, 2 * D + V), 2)
+    k0 = torch.zeros(D)
+    k0[5] = 1.0
+    qkv[0, D:2 * D] = k0
+    qkv[0, 2 * D:] = 3.0
+    qkv[-1, :D] = k0
+    gates = torch.full((T, 1), -20.0)
+    gates[0] = 20.0
+    decay = torch.zeros(T, D)
+    a_log, dt_bias = torch.zeros(1), torch.full((D,), -12.0)
+
+    def read(rows, gate_rows, cuts):
+        state = torch.zeros((1, D * V), dtype=torch.float32, device=DEV)
+        at, last = 0, None
+        for n in cuts:
+            out = torch.empty((n, H, V), dtype=torch.float32, device=DEV)
+            ops.delta_rule(rows[at:at + n].contiguous().to(DEV), gate_rows[at:at + n].contiguous().to(DEV), 0, 0,
+                           a_log.to(DEV), dt_bias.to(DEV), state, 0, i32([0, n]), i32([0]), out, H, G, D, V,
+                           decay=decay[at:at + n].contiguous().to(DEV), per_channel=True)
+            at, last = at + n, out[-1, 0].cpu()
+        return last
+
+    got = read(qkv, gates, [T])
+    assert float((got - 3.0 * D ** -0.5).abs().max()) < 0.02, got            # q = k0 / sqrt(dim) reads v0 back
+    close(read(qkv, gates, [900, 2, 498]), got, torch.float32, "in three steps")
+    silent = gates.clone()
+    silent[0] = -20.0
+    assert float(read(qkv, silent, [T]).abs().max()) < 0.01
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_read_out_with_a_sigmoid_gate(dtype):
     ops = gpu_ops()
