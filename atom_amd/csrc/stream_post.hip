@@ -5,6 +5,7 @@
 //                     stream's new rows in the step's type for the products that read them next
 //   rmsnorm_rows      norm of chosen float32 rows, written in another type
 //   cast_rows         float32 rows in another type
+//   bias_rows         y[r, :] += bias for float32 rows
 //   token_gate        gelu_tanh(a[t, j]) * table[id[t], col_off + j]
 //   embedding_bigram  table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets], float32; a request's
 //                     first token takes row `buckets`; the previous token of a request's next token is kept per
@@ -204,6 +205,38 @@ ATOM_EXPORT int atom_cast_rows(const float* x, void* out, int out_dtype, long n,
   if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
   ATOM_DISPATCH_DTYPE(out_dtype, hipLaunchKernelGGL((cast_rows_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, x,
                                                      (T*)out, (size_t)n));
+  return launch_status();
+}
+
+// y[r, :] += bias for float32 rows (the bias of a library product whose output stays float32); 16-byte accesses
+// where the width allows them.
+__global__ void bias_rows_kernel(float* __restrict__ y, const float* __restrict__ bias, int width, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < total) y[idx] += bias[idx % width];
+}
+
+__global__ void bias_rows_vec_kernel(float4* __restrict__ y, const float4* __restrict__ bias, int quads, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  float4 v = y[idx];
+  const float4 b = bias[idx % quads];
+  v.x += b.x; v.y += b.y; v.z += b.z; v.w += b.w;
+  y[idx] = v;
+}
+
+ATOM_EXPORT int atom_bias_rows(float* y, const float* bias, int rows, int width, hipStream_t stream) {
+  if (rows < 0 || width <= 0 || y == nullptr || bias == nullptr) return ATOM_BAD_SHAPE;
+  size_t total = (size_t)rows * width;
+  if (total == 0) return ATOM_OK;
+  const bool vec = width % 4 == 0 && (uintptr_t)y % 16 == 0 && (uintptr_t)bias % 16 == 0;
+  if (vec) total /= 4;
+  const size_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffu) return ATOM_TOO_LARGE;
+  if (vec)
+    hipLaunchKernelGGL(bias_rows_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (float4*)y, (const float4*)bias,
+                       width / 4, total);
+  else
+    hipLaunchKernelGGL(bias_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, y, bias, width, total);
   return launch_status();
 }
 

@@ -195,7 +195,7 @@ class HipKernels:
                    "atom_experts_grouped", "atom_experts_grouped_tiles", "atom_experts_grouped_supports",
                    "atom_heads_gemm_mfma", "atom_heads_gemm_mfma_supports", "atom_rmsnorm_post", "atom_rmsnorm_rows",
                    "atom_cast_rows", "atom_token_gate", "atom_embedding_bigram", "atom_rglru_scan",
-                   "atom_keys_as_values_write", "atom_sigmoid_gate"):
+                   "atom_keys_as_values_write", "atom_sigmoid_gate", "atom_bias_rows"):
             getattr(self.lib, fn).restype = ctypes.c_int
         self.allow_library_gemm = True
         # bfloat16 products of few rows run this library's own weight-streaming kernels: up to 64 rows, and
@@ -814,7 +814,7 @@ class HipKernels:
             # same precision whatever the number of rows, and a bias is added before anything is rounded
             y = torch.mm(x, weight.t(), out_dtype=torch.float32)
             if bias is not None:
-                y += bias
+                self._done("bias_rows", self.lib.atom_bias_rows(_ptr(y), _ptr(bias), m, n, self._stream()))
             return y if out_dtype == torch.float32 else y.to(out_dtype)
         y = torch.empty((m, n), dtype=out_dtype, device=x.device)
         self._done("gemm_f32", self.lib.atom_gemm_f32(
