@@ -344,7 +344,8 @@ ATOM_EXPORT int atom_latent_attention(const void* q_abs, const void* pages, void
 // ------------------------------------------------------------------ the per-head products on the matrix cores
 //
 // The same product as heads_gemm with bfloat16 weights, for many rows: the head's weight rows are the A operand and
-// the tokens the B operand, both read straight from memory (a float32 input is rounded to bfloat16 on the way), so a
+// the tokens the B operand, both read straight from memory (a float32 input is rounded to bfloat16 on the way, or,
+// where the product is to be the float32 one, split into three bfloat16 pieces that are multiplied one by one), so a
 // lane ends up with four consecutive columns of one token.  A block of 2 x 2 waves owns 64 tokens x 64 columns.
 // Needs k % 8 == 0 and offsets and strides of x that keep its 8-element pieces aligned.
 
@@ -369,7 +370,29 @@ __device__ __forceinline__ hg_bf16x8 hg_load8(const float* p, bool ok) {
   return out;
 }
 
-template <typename TX, typename TY>
+// A float32 input in three bfloat16 pieces, x = hi + mid + lo exactly (3 x 8 bits of mantissa): the products of each
+// piece with a bfloat16 weight are exact in float32 and the matrix cores add them in float32, so the three products
+// together are the float32 product, at three matrix instructions instead of 32 multiply-adds a lane.
+__device__ __forceinline__ void hg_load8_split(const float* p, bool ok, hg_bf16x8* hi, hg_bf16x8* mid, hg_bf16x8* lo) {
+  const hg_bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  *hi = *mid = *lo = zero;
+  if (ok) {
+    const hg_f32x4 a = *reinterpret_cast<const hg_f32x4*>(p), b = *reinterpret_cast<const hg_f32x4*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float v = i < 4 ? a[i] : b[i - 4];
+      const __bf16 h = static_cast<__bf16>(v);
+      const float r1 = v - static_cast<float>(h);
+      const __bf16 m = static_cast<__bf16>(r1);
+      const float r2 = r1 - static_cast<float>(m);
+      (*hi)[i] = h;
+      (*mid)[i] = m;
+      (*lo)[i] = static_cast<__bf16>(r2);
+    }
+  }
+}
+
+template <typename TX, typename TY, bool SPLIT = false>
 __global__ void __launch_bounds__(256)
 heads_gemm_mfma_kernel(const TX* __restrict__ x, long ldx, long hsx, const bf16_t* __restrict__ w, TY* __restrict__ y,
                        long ldy, long hsy, const float* __restrict__ gate, long ldg, int m, int n, int k, float alpha) {
@@ -402,15 +425,24 @@ heads_gemm_mfma_kernel(const TX* __restrict__ x, long ldx, long hsx, const bf16_
     const int kk = k0 + 8 * g;
     const bool kok = kk < k;
     hg_bf16x8 xb[2], wa[2];
+    [[maybe_unused]] hg_bf16x8 xm[2], xl[2];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) xb[rt] = hg_load8(xrow[rt] + kk, kok && rok[rt]);
+    for (int rt = 0; rt < 2; ++rt) {
+      if constexpr (SPLIT) hg_load8_split(xrow[rt] + kk, kok && rok[rt], &xb[rt], &xm[rt], &xl[rt]);
+      else xb[rt] = hg_load8(xrow[rt] + kk, kok && rok[rt]);
+    }
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct) wa[ct] = hg_load8(wrow[ct] + kk, kok && cok[ct]);
 #pragma unroll
     for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-      for (int rt = 0; rt < 2; ++rt)
+      for (int rt = 0; rt < 2; ++rt) {
+        if constexpr (SPLIT) {   // the small pieces first
+          acc[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ct], xl[rt], acc[ct][rt], 0, 0, 0);
+          acc[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ct], xm[rt], acc[ct][rt], 0, 0, 0);
+        }
         acc[ct][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[ct], xb[rt], acc[ct][rt], 0, 0, 0);
+      }
   }
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
@@ -436,8 +468,9 @@ ATOM_EXPORT int atom_heads_gemm_mfma_supports(int x_dtype, int w_dtype, long x_o
 
 ATOM_EXPORT int atom_heads_gemm_mfma(const void* x, int x_dtype, long ldx, long hsx, const void* w, void* y, int y_dtype,
                                      long ldy, long hsy, const float* gate, long ldg, int heads, int m, int n, int k,
-                                     float alpha, hipStream_t stream) {
+                                     float alpha, int split, hipStream_t stream) {
   if (m < 0 || n <= 0 || k <= 0 || heads <= 0 || heads > 65535 || (k % 8)) return ATOM_BAD_SHAPE;
+  if (split && x_dtype != ATOM_F32) return ATOM_UNSUPPORTED;   // only a float32 input has pieces to split into
   if (x == nullptr || w == nullptr || y == nullptr) return ATOM_BAD_SHAPE;
   if ((unsigned)x_dtype > 1u || (unsigned)y_dtype > 1u) return ATOM_BAD_DTYPE;
   if (m == 0) return ATOM_OK;
@@ -446,6 +479,15 @@ ATOM_EXPORT int atom_heads_gemm_mfma(const void* x, int x_dtype, long ldx, long 
 #define LAUNCH(TX, TY)                                                                                            \
   hipLaunchKernelGGL((heads_gemm_mfma_kernel<TX, TY>), grid, block, 0, stream, (const TX*)x, ldx, hsx,           \
                      (const bf16_t*)w, (TY*)y, ldy, hsy, gate, ldg, m, n, k, alpha)
+  if (split) {
+    if (y_dtype == ATOM_F32)
+      hipLaunchKernelGGL((heads_gemm_mfma_kernel<float, float, true>), grid, block, 0, stream, (const float*)x, ldx, hsx,
+                         (const bf16_t*)w, (float*)y, ldy, hsy, gate, ldg, m, n, k, alpha);
+    else
+      hipLaunchKernelGGL((heads_gemm_mfma_kernel<float, bf16_t, true>), grid, block, 0, stream, (const float*)x, ldx, hsx,
+                         (const bf16_t*)w, (bf16_t*)y, ldy, hsy, gate, ldg, m, n, k, alpha);
+    return launch_status();
+  }
   switch (x_dtype * 2 + y_dtype) {
     case 0: LAUNCH(float, float); break;
     case 1: LAUNCH(float, bf16_t); break;

@@ -224,6 +224,7 @@ class HipKernels:
         # products on the matrix cores; below, every pair reads its expert's rows itself
         self.grouped_experts_from = 64
         self.heads_mfma_from = 1       # rows from which the per-head products run on the matrix cores
+        self.heads_split_from = 9      # ... and from which the exact ones do, on a float32 input's three pieces
         self._ws: dict[str, torch.Tensor] = {}
         self._extensions: dict = {}
         self._zeroed: dict[str, torch.Tensor] = {}   # workspaces that every kernel leaves all zero
@@ -986,7 +987,9 @@ class HipKernels:
         """One small product per head: ``y[t, h, :n] = alpha * x[t, h, :k] @ weight[h].T`` (times
         ``sigmoid(gate[t, h])`` when given), with ``x`` and ``y`` addressed as flat arrays: element (t, h, i) of x
         sits at ``x_offset + t * ldx + h * hsx + i``.  ``weight`` is [heads, n, k].  ``exact``: a float32 input is
-        multiplied as it is (float32 multiply-adds), not rounded for the matrix cores."""
+        multiplied as it is, not rounded for the matrix cores: float32 multiply-adds for few rows or float32
+        weights, and for many rows with bfloat16 weights the matrix cores on the input's three bfloat16 pieces,
+        whose products with a bfloat16 weight are exact."""
         self._check("per-head input", x, (torch.float32, torch.bfloat16))
         self._check("per-head weight", weight, (torch.float32, torch.bfloat16), (heads, n, k))
         self._check("per-head out", y, (torch.float32, torch.bfloat16))
@@ -1003,14 +1006,15 @@ class HipKernels:
             gp = ctypes.c_void_p(gate.data_ptr() + 4 * gate_offset)
         xp = ctypes.c_void_p(x.data_ptr() + x.element_size() * x_offset)
         yp = ctypes.c_void_p(y.data_ptr() + y.element_size() * y_offset)
-        if (weight.dtype == torch.bfloat16 and m >= self.heads_mfma_from and not (exact and x.dtype == torch.float32)
+        split = bool(exact and x.dtype == torch.float32)
+        if (weight.dtype == torch.bfloat16 and m >= (self.heads_split_from if split else self.heads_mfma_from)
                 and self.lib.atom_heads_gemm_mfma_supports(
                 self._code(x), BF16, ctypes.c_long(x_offset), ctypes.c_long(ldx), ctypes.c_long(hsx), k)):
             # many rows: the same product on the matrix cores (a float32 input is rounded to bfloat16 on the way in)
             self._done("heads_gemm_mfma", self.lib.atom_heads_gemm_mfma(
                 xp, self._code(x), ctypes.c_long(ldx), ctypes.c_long(hsx), _ptr(weight), yp, self._code(y),
                 ctypes.c_long(ldy), ctypes.c_long(hsy), gp, ctypes.c_long(ldg), heads, m, n, k, ctypes.c_float(alpha),
-                self._stream()))
+                int(split), self._stream()))
             return y
         self._done("heads_gemm", self.lib.atom_heads_gemm(
             xp, self._code(x), ctypes.c_long(ldx), ctypes.c_long(hsx), _ptr(weight), self._code(weight), yp,
