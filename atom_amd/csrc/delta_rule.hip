@@ -159,7 +159,8 @@ delta_prepare_kernel(float* __restrict__ qkv, int channels, float* __restrict__ 
 }
 
 constexpr int kRun = 16;   // tokens whose q, k and gates are staged at once
-constexpr int kDPL = 16;   // entries of a column of S that one lane holds
+constexpr int kDPL = 16;   // entries of a column of S that one lane holds (8 for heads of 65 to 128 key channels, whose
+                           // columns then spread over 16 lanes: half the multiply-adds a token and wave, twice the waves)
 
 // qkv [T, channels] float32 after convolution and SiLU: q heads (kv_heads x dim) | k heads | v heads (heads x vdim).
 // ab [T, ld_ab] float32: the raw decay inputs at a_off and the raw beta inputs at b_off, one per head.
@@ -169,7 +170,7 @@ constexpr int kDPL = 16;   // entries of a column of S that one lane holds
 //
 // CHANNEL: the decay is one number per head and key channel (row of S): dec holds heads x dim raw inputs a token at
 // a_off, dt_bias heads x dim entries, and a run's decays are staged like its q and k rows.
-template <int LPC, bool CHANNEL>
+template <int LPC, bool CHANNEL, int DPL = kDPL>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __restrict__ ab, int ld_ab,
                   const float* __restrict__ dec, int ld_dec, int a_off,
@@ -177,7 +178,7 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
                   float* __restrict__ state, long slot_stride, long state_off, const int* __restrict__ cu_seqlens,
                   const int* __restrict__ slot_of_seq, float* __restrict__ out, int heads, int kv_heads, int dim,
                   int vdim) {
-  constexpr int DMAX = kDPL * LPC;
+  constexpr int DMAX = DPL * LPC;
   __shared__ __attribute__((aligned(16))) float qs[kRun][DMAX];
   __shared__ __attribute__((aligned(16))) float ks[kRun][DMAX];
   __shared__ __attribute__((aligned(16))) float gv[CHANNEL ? kRun : 1][DMAX];   // CHANNEL: a run's decays per key channel
@@ -196,10 +197,10 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     return;
   }
   float* sp = state + (size_t)slot * slot_stride + state_off + (size_t)head * dim * vdim;   // [dim, vdim]
-  float S[kDPL];
+  float S[DPL];
 #pragma unroll
-  for (int j = 0; j < kDPL; ++j) {
-    const int i = sub * kDPL + j;
+  for (int j = 0; j < DPL; ++j) {
+    const int i = sub * DPL + j;
     S[j] = (live && i < dim) ? sp[(size_t)i * vdim + col] : 0.f;
   }
   const int k_off = kv_heads * dim, v_off = 2 * kv_heads * dim;
@@ -264,13 +265,13 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     if (t0 + kRun < end) load_run(t0 + kRun);
     // a token's k and q entries are read from LDS one token ahead of their use, so that the chain below never
     // waits for them
-    float kc[kDPL], qc[kDPL], kn[kDPL], qn[kDPL];
-    float gc[CHANNEL ? kDPL : 1], gn[CHANNEL ? kDPL : 1];
+    float kc[DPL], qc[DPL], kn[DPL], qn[DPL];
+    float gc[CHANNEL ? DPL : 1], gn[CHANNEL ? DPL : 1];
 #pragma unroll
-    for (int e = 0; e < kDPL; ++e) {
-      kc[e] = ks[0][sub * kDPL + e];
-      qc[e] = qs[0][sub * kDPL + e];
-      if constexpr (CHANNEL) gc[e] = gv[0][sub * kDPL + e];
+    for (int e = 0; e < DPL; ++e) {
+      kc[e] = ks[0][sub * DPL + e];
+      qc[e] = qs[0][sub * DPL + e];
+      if constexpr (CHANNEL) gc[e] = gv[0][sub * DPL + e];
     }
     // A whole run is walked without a test per token: the registers that hold the next token's entries then simply
     // become the current ones, with no copies (a test per token makes every hand-over a set of moves).
@@ -284,15 +285,15 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
 
       if (j + 1 < kRun) {
 #pragma unroll
-        for (int e = 0; e < kDPL; ++e) {
-          kn[e] = ks[j + 1][sub * kDPL + e];
-          qn[e] = qs[j + 1][sub * kDPL + e];
-          if constexpr (CHANNEL) gn[e] = gv[j + 1][sub * kDPL + e];
+        for (int e = 0; e < DPL; ++e) {
+          kn[e] = ks[j + 1][sub * DPL + e];
+          qn[e] = qs[j + 1][sub * DPL + e];
+          if constexpr (CHANNEL) gn[e] = gv[j + 1][sub * DPL + e];
         }
       }
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int e = 0; e < kDPL; ++e) {
+      for (int e = 0; e < DPL; ++e) {
         if constexpr (CHANNEL) S[e] *= gc[e]; else S[e] *= g;
         part[e & 3] = fmaf(S[e], kc[e], part[e & 3]);
       }
@@ -300,14 +301,14 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
       const float u = beta * (v - dot);
       part[0] = part[1] = part[2] = part[3] = 0.f;
 #pragma unroll
-      for (int e = 0; e < kDPL; ++e) {
+      for (int e = 0; e < DPL; ++e) {
         S[e] = fmaf(kc[e], u, S[e]);
         part[e & 3] = fmaf(S[e], qc[e], part[e & 3]);
       }
       const float o = group_sum<LPC>((part[0] + part[1]) + (part[2] + part[3]));
       if (live && sub == 0) out[((size_t)(t0 + j) * heads + head) * vdim + col] = o;
 #pragma unroll
-      for (int e = 0; e < kDPL; ++e) {
+      for (int e = 0; e < DPL; ++e) {
         kc[e] = kn[e];
         qc[e] = qn[e];
         if constexpr (CHANNEL) gc[e] = gn[e];
@@ -319,8 +320,8 @@ delta_rule_kernel(const float* __restrict__ qkv, int channels, const float* __re
     else walk(std::false_type{});
   }
 #pragma unroll
-  for (int j = 0; j < kDPL; ++j) {
-    const int i = sub * kDPL + j;
+  for (int j = 0; j < DPL; ++j) {
+    const int i = sub * DPL + j;
     if (live && i < dim) sp[(size_t)i * vdim + col] = S[j];
   }
 }
@@ -344,6 +345,8 @@ ATOM_EXPORT int atom_delta_rule(float* qkv, int tokens, int channels, const floa
                      dt_bias, heads, kv_heads, dim, per_channel ? dim : 1);
   int lpc = 1;
   while (lpc * kDPL < dim) lpc *= 2;
+  const bool narrow = dim > 64 && dim <= 128;   // 16 lanes of 8 entries instead of 8 lanes of 16
+  if (narrow) lpc = 16;
   const int cols = 256 / lpc;
   dim3 grid(heads, num_seqs, (vdim + cols - 1) / cols), block(256);
   if (grid.z > 65535) return ATOM_TOO_LARGE;
@@ -358,6 +361,17 @@ ATOM_EXPORT int atom_delta_rule(float* qkv, int tokens, int channels, const floa
       LAUNCH_AS(L, false);         \
     }                              \
   } while (0)
+  if (narrow) {
+    if (per_channel)
+      hipLaunchKernelGGL((delta_rule_kernel<16, true, 8>), grid, block, 0, stream, qkv, channels, ab, ld_ab, dec, ld_dec,
+                         a_off, b_off, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim,
+                         vdim);
+    else
+      hipLaunchKernelGGL((delta_rule_kernel<16, false, 8>), grid, block, 0, stream, qkv, channels, ab, ld_ab, dec, ld_dec,
+                         a_off, b_off, state, slot_stride, state_off, cu_seqlens, slot_of_seq, out, heads, kv_heads, dim,
+                         vdim);
+    return launch_status();
+  }
   switch (lpc) {
     case 1: LAUNCH(1); break;
     case 2: LAUNCH(2); break;
