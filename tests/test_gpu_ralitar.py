@@ -596,3 +596,27 @@ def test_trace_program(dtype, tmp_path):
     results = replay.run_program(rt.folder("V"), dtype, steps, str(tmp_path / "out"), replay.peak_tokens(steps, 64),
                                  rt.CONFIGS["V"]["vocab"])
     _check(steps, results, requests, "V", dtype, f"program/{dtype}")
+
+
+def test_command_line():
+    """``python -m atom_amd.examples.simple_inference`` on a Ralitar folder: the registry picks the design from
+    config.json; greedy completions are the plain implementation's."""
+    import random
+    import re
+    import subprocess
+    import sys
+
+    cmd = [sys.executable, "-m", "atom_amd.examples.simple_inference", "--model", rt.folder("V"), "--temperature", "0",
+           "--max-tokens", "6", "--block_size", "16", "--num-kvcache-blocks", "32", "--max-num-seqs", "4", "--dtype", "fp32",
+           "--max-model-len", "256", "--seed", "3"]
+    res = subprocess.run(cmd, cwd=replay.ROOT, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert res.stdout.count("Completion:") == 3 and res.stdout.count("finish_reason=max_tokens") == 3
+    rng = random.Random(3)
+    prompts = [[rng.randrange(rt.CONFIGS["V"]["vocab"]) for _ in range(n)] for n in (5, 17, 33)]
+    shown = [eval(m) for m in re.findall(r"Completion: (\[.*?\])", res.stdout)]
+    for prompt, out in zip(prompts, shown):
+        tokens = list(prompt)
+        for token in out:
+            assert token == int(rt.oracle("V", tokens)[-1].argmax())
+            tokens.append(token)
